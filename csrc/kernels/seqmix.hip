@@ -38,31 +38,50 @@ __device__ __forceinline__ float silu_f(float z) { return z / (1.f + expf(-z)); 
 // ---------------------------------------------------------------- rms_rows
 template <typename TI, typename TO>
 __global__ void __launch_bounds__(256) rms_rows_kernel(const TI* __restrict__ x, long ldx, const float* __restrict__ w,
-                                                       TO* __restrict__ y, long ldy, int rows, int n, float eps) {
-  const int row = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
-  if (row >= rows) return;
-  const TI* xr = x + (long)row * ldx;
+                                                       TO* __restrict__ y, long ldy, int rows, int n, float eps,
+                                                       int groups) {
+  // a wave per (row, part): `groups` equal consecutive parts of a row, each by its own root mean square
+  const int unit = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+  if (unit >= rows * groups) return;
+  const int row = unit / groups, c0 = (unit % groups) * n;
+  const TI* xr = x + (long)row * ldx + c0;
   float s = 0.f;
   for (int i = lane; i < n; i += 64) { const float v = ldf(xr + i); s += v * v; }
   s = wave_sum(s);
   const float r = 1.f / sqrtf(s / (float)n + eps);
-  TO* yr = y + (long)row * ldy;
-  for (int i = lane; i < n; i += 64) stf(yr + i, ldf(xr + i) * r * (w ? w[i] : 1.f));
+  TO* yr = y + (long)row * ldy + c0;
+  for (int i = lane; i < n; i += 64) stf(yr + i, ldf(xr + i) * r * (w ? w[c0 + i] : 1.f));
 }
 
 // ---------------------------------------------------------------- norm_resadd
 template <typename T>
 __global__ void __launch_bounds__(256) norm_resadd_kernel(const T* __restrict__ y, long ldy, const float* __restrict__ w,
-                                                          float* __restrict__ x, T* __restrict__ xl, int H, float eps) {
+                                                          float* __restrict__ x, T* __restrict__ xl, int H, float eps,
+                                                          int groups, const float* __restrict__ bias) {
   __shared__ float red[16];
   const long row = blockIdx.x;
   const T* yr = y + row * ldy;
-  float s = 0.f;
-  for (int i = threadIdx.x; i < H; i += 256) { const float v = ldf(yr + i); s += v * v; }
-  const float r = 1.f / sqrtf(block_sum(s, red) / (float)H + eps);
   float* xr = x + row * (long)H;
+  if (groups > 1) {   // a wave per part of the row: no workgroup barrier
+    const int n = H / groups, lane = threadIdx.x & 63;
+    for (int g = threadIdx.x >> 6; g < groups; g += 4) {
+      const int c0 = g * n;
+      float s = 0.f;
+      for (int i = lane; i < n; i += 64) { const float v = ldf(yr + c0 + i) + (bias ? bias[c0 + i] : 0.f); s += v * v; }
+      const float r = 1.f / sqrtf(wave_sum(s) / (float)n + eps);
+      for (int i = lane; i < n; i += 64) {
+        const float v = xr[c0 + i] + (ldf(yr + c0 + i) + (bias ? bias[c0 + i] : 0.f)) * r * w[c0 + i];
+        xr[c0 + i] = v;
+        if (xl) stf(xl + row * (long)H + c0 + i, v);
+      }
+    }
+    return;
+  }
+  float s = 0.f;
+  for (int i = threadIdx.x; i < H; i += 256) { const float v = ldf(yr + i) + (bias ? bias[i] : 0.f); s += v * v; }
+  const float r = 1.f / sqrtf(block_sum(s, red) / (float)H + eps);
   for (int i = threadIdx.x; i < H; i += 256) {
-    const float v = xr[i] + ldf(yr + i) * r * w[i];
+    const float v = xr[i] + (ldf(yr + i) + (bias ? bias[i] : 0.f)) * r * w[i];
     xr[i] = v;
     if (xl) stf(xl + row * (long)H + i, v);
   }
@@ -657,26 +676,29 @@ __global__ void __launch_bounds__(256) dense_gate_kernel(const int* __restrict__
   if (f32) { call_f32; } else { call_u16; }
 
 extern "C" int dllm_rms_rows(const void* x, long ldx, int x_f32, const float* w, void* y, long ldy, int y_f32, int rows,
-                             int n, float eps, hipStream_t st) {
+                             int n, float eps, int groups, hipStream_t st) {
   if (rows <= 0 || n <= 0) return rows == 0 ? 0 : -1;
-  const dim3 g((rows + 3) / 4), b(256);
+  if (groups < 1 || n % groups) return -1;
+  n /= groups;     // the kernel's rows are the parts
+  const dim3 g((rows * groups + 3) / 4), b(256);
   if (x_f32 && y_f32)
-    hipLaunchKernelGGL((rms_rows_kernel<float, float>), g, b, 0, st, (const float*)x, ldx, w, (float*)y, ldy, rows, n, eps);
+    hipLaunchKernelGGL((rms_rows_kernel<float, float>), g, b, 0, st, (const float*)x, ldx, w, (float*)y, ldy, rows, n, eps, groups);
   else if (x_f32)
-    hipLaunchKernelGGL((rms_rows_kernel<float, u16>), g, b, 0, st, (const float*)x, ldx, w, (u16*)y, ldy, rows, n, eps);
+    hipLaunchKernelGGL((rms_rows_kernel<float, u16>), g, b, 0, st, (const float*)x, ldx, w, (u16*)y, ldy, rows, n, eps, groups);
   else if (y_f32)
-    hipLaunchKernelGGL((rms_rows_kernel<u16, float>), g, b, 0, st, (const u16*)x, ldx, w, (float*)y, ldy, rows, n, eps);
+    hipLaunchKernelGGL((rms_rows_kernel<u16, float>), g, b, 0, st, (const u16*)x, ldx, w, (float*)y, ldy, rows, n, eps, groups);
   else
-    hipLaunchKernelGGL((rms_rows_kernel<u16, u16>), g, b, 0, st, (const u16*)x, ldx, w, (u16*)y, ldy, rows, n, eps);
+    hipLaunchKernelGGL((rms_rows_kernel<u16, u16>), g, b, 0, st, (const u16*)x, ldx, w, (u16*)y, ldy, rows, n, eps, groups);
   return (int)hipGetLastError();
 }
 
 extern "C" int dllm_norm_resadd(const void* y, long ldy, int f32, const float* w, float* x, void* xl, int rows, int H,
-                                float eps, hipStream_t st) {
+                                float eps, int groups, const float* bias, hipStream_t st) {
   if (rows <= 0) return rows == 0 ? 0 : -1;
+  if (groups < 1 || H % groups) return -1;
   BY_T(f32,
-       hipLaunchKernelGGL(norm_resadd_kernel<u16>, dim3(rows), dim3(256), 0, st, (const u16*)y, ldy, w, x, (u16*)xl, H, eps),
-       hipLaunchKernelGGL(norm_resadd_kernel<float>, dim3(rows), dim3(256), 0, st, (const float*)y, ldy, w, x, (float*)xl, H, eps))
+       hipLaunchKernelGGL(norm_resadd_kernel<u16>, dim3(rows), dim3(256), 0, st, (const u16*)y, ldy, w, x, (u16*)xl, H, eps, groups, bias),
+       hipLaunchKernelGGL(norm_resadd_kernel<float>, dim3(rows), dim3(256), 0, st, (const float*)y, ldy, w, x, (float*)xl, H, eps, groups, bias))
   return (int)hipGetLastError();
 }
 

@@ -104,8 +104,13 @@ class MixerSpec:
     dim, vdim, decay per head, rot), ``latent_attention`` (heads, dim, rot_dim, vdim, kv_rank,
     q_rank, scale, rot), ``delta`` (gated delta rule: heads, kv_heads, dim, vdim, conv),
     ``softmax_attention`` (grouped-query, paged: heads, kv_heads, dim, vdim, scale, rot),
-    ``lightning`` (heads, dim, vdim, decay per head) or ``parallel`` (``left`` and ``right`` mixers
-    over the same input)."""
+    ``lightning`` (heads, dim, vdim, decay per head), ``parallel`` (``left`` and ``right`` mixers
+    over the same input), ``diff_attention`` (two softmax maps per head over shared values, combined
+    as a1 - lambda a2: heads, kv_heads, dim, vdim, scale, rot, ``window`` keys seen (0: all),
+    ``diff``, ``kv_from`` = the layer whose cached keys / values it reads instead of its own),
+    ``mamba2`` (scalar decay per head: heads, vdim, state, groups of heads sharing B / C, conv,
+    norm_groups of the gated output norm) or ``mlstm`` (matrix memory with exponential gates:
+    heads, dim, vdim, gate_cap)."""
     kind: str
     inner: int = 0
     state: int = 0
@@ -123,6 +128,12 @@ class MixerSpec:
     kv_heads: int = 0
     left: Optional["MixerSpec"] = None
     right: Optional["MixerSpec"] = None
+    window: int = 0
+    diff: float = 0.0
+    kv_from: Optional[int] = None
+    groups: int = 1
+    norm_groups: int = 1
+    gate_cap: float = 0.0
 
     @property
     def parts(self) -> Tuple["MixerSpec", ...]:
@@ -130,27 +141,39 @@ class MixerSpec:
 
     @property
     def recurrent(self) -> bool:
-        return any(p.kind in ("mamba1", "retention", "delta", "lightning") for p in self.parts)
+        return any(p.kind in ("mamba1", "retention", "delta", "lightning", "mamba2", "mlstm") for p in self.parts)
 
     @property
     def paged(self) -> bool:
-        return any(p.kind in ("latent_attention", "softmax_attention") for p in self.parts)
+        return any(p.kind in ("latent_attention", "softmax_attention") or
+                   (p.kind == "diff_attention" and p.kv_from is None) for p in self.parts)
 
 
 @dataclass(frozen=True)
 class MoESpec:
     """Routed experts (``ff`` wide, ``top`` of ``experts`` per token, weights times ``scale``) and an
-    optional shared expert (``shared_ff`` > 0) that every token runs."""
+    optional shared expert (``shared_ff`` > 0) that every token runs.  ``act``: ``relu2``
+    (W_down relu(W_up x)^2) or ``swiglu`` (W_down (silu(W_gate x) * W_up x)).  ``score``:
+    ``softmax`` (the chosen experts' weights renormalised) or ``sigmoid`` (weights = the chosen
+    scores as they are); with ``group_count`` > 1 the experts form that many groups of neighbours,
+    a group scores the sum of its two best experts and only the ``group_keep`` best groups' experts
+    can be chosen."""
     experts: int
     top: int
     scale: float
     ff: int
     shared_ff: int = 0
+    act: str = "relu2"
+    score: str = "softmax"
+    group_count: int = 1
+    group_keep: int = 1
 
 
 @dataclass(frozen=True)
 class DenseSpec:
-    """One dense feed-forward ``W_down act(W_up x)``, ``ff`` wide; ``act``: ``gelu`` (the erf form)."""
+    """One dense feed-forward ``W_down act(W_up x)``, ``ff`` wide; ``act``: ``gelu`` (the erf form) or
+    ``polynorm`` (a N(z) + b N(z^2) + c N(z^3) + e with learned a, b, c, e and N the scaling of a
+    token's ff values to unit RMS)."""
     ff: int
     act: str = "gelu"
 
@@ -178,6 +201,11 @@ class HybridConfig:
     pre_norm: bool = False
     # what a layer hands on is a learned weighted sum of the embedding output and every layer result so far
     depth_average: bool = False
+    # the model's norms (after each sublayer, before the head) split the vector into this many equal
+    # consecutive parts, each divided by its own root mean square
+    norm_groups: int = 1
+    # logits <- cap * tanh(logits / cap) (0: none)
+    logit_softcap: float = 0.0
 
     @property
     def n_layers(self) -> int:
@@ -208,12 +236,21 @@ class HybridConfig:
                 elif m.kind == "delta":
                     c = 2 * m.kv_heads * m.dim + m.heads * m.vdim
                     n += c * (H + m.conv) + 2 * m.heads * (H + 1) + m.vdim + 2 * m.heads * m.vdim * H
+                elif m.kind == "diff_attention":
+                    n += 2 * m.heads * m.dim * (H + 1) + 5 * m.dim + m.heads * m.vdim * H + H
+                    if m.kv_from is None:
+                        n += (2 * m.kv_heads * m.dim + m.kv_heads * m.vdim) * (H + 1) + m.dim
+                elif m.kind == "mamba2":
+                    inner, bc = m.heads * m.vdim, 2 * m.groups * m.state
+                    n += (2 * inner + bc + m.heads) * H + (inner + bc) * (m.conv + 1) + 3 * m.heads + inner + H * inner
+                elif m.kind == "mlstm":
+                    n += 2 * m.heads * m.dim * H + 3 * m.heads * m.vdim * H + m.heads * m.vdim + 2 * m.heads * (H + 1)
             n += H * (2 if self.pre_norm else 1)
             if isinstance(L.mlp, MoESpec):
                 f = L.mlp
-                n += H + f.experts * (H + 2 * f.ff * H) + 2 * f.shared_ff * H
+                n += H + f.experts * (H + (3 if f.act == "swiglu" else 2) * f.ff * H) + 2 * f.shared_ff * H
             elif isinstance(L.mlp, DenseSpec):
-                n += 2 * H + 2 * L.mlp.ff * H
+                n += 2 * H + 2 * L.mlp.ff * H + (4 if L.mlp.act == "polynorm" else 0)
         if self.depth_average:
             n += sum(i + 2 for i in range(len(self.layers)))
         return n
@@ -292,8 +329,65 @@ def sedopel_config(raw: dict, name: str = "sedopel") -> HybridConfig:
                         rms_eps=float(raw["norm"]["eps"]), pre_norm=True, depth_average=True)
 
 
+def pebodra_config(raw: dict, name: str = "pebodra") -> HybridConfig:
+    """A Pebodra config.json: ``layers`` (type ``attention``, ``mamba2`` or ``mlstm``, mixer sizes,
+    mlp ``dense`` / ``moe`` or null), ``norm.eps``, ``norm.groups``, ``logit_softcap``, ``vocab``,
+    ``width``.  An attention mixer with ``kv_from`` reads that layer's cached keys and values."""
+    W = int(raw["width"])
+    layers = []
+    for i, L in enumerate(raw["layers"]):
+        m, kind = L["mixer"], L["type"]
+        if kind == "attention":
+            mask = m.get("mask") or {}
+            src = m.get("kv_from")
+            mix = MixerSpec("diff_attention", heads=int(m["heads"]), kv_heads=int(m.get("kv_heads", m["heads"])),
+                            dim=int(m["dim"]), vdim=int(m["vdim"]), scale=float(m["scale"]), rot=_rope(m.get("rot")),
+                            window=int(mask.get("size", 0)), diff=float(m["diff"]),
+                            kv_from=None if src is None else int(src))
+            if mix.heads % mix.kv_heads:
+                raise ValueError("heads must be a multiple of kv_heads")
+            if mix.kv_from is not None:
+                if not 0 <= mix.kv_from < i or layers[mix.kv_from].mixer.kind != "diff_attention" \
+                        or layers[mix.kv_from].mixer.kv_from is not None:
+                    raise ValueError(f"layer {i}: kv_from must name an earlier attention layer with keys of its own")
+                src_m = layers[mix.kv_from].mixer
+                if (src_m.kv_heads, src_m.dim, src_m.vdim) != (mix.kv_heads, mix.dim, mix.vdim):
+                    raise ValueError(f"layer {i}: the layer it takes keys and values from has other head sizes")
+        elif kind == "mamba2":
+            mix = MixerSpec(kind, heads=int(m["heads"]), vdim=int(m["vdim"]), state=int(m["state"]),
+                            groups=int(m.get("groups", 1)), conv=int(m["conv"]), norm_groups=int(m.get("norm_groups", 1)))
+            if mix.heads % mix.groups or (mix.heads * mix.vdim) % mix.norm_groups:
+                raise ValueError("heads must be a multiple of groups, heads * vdim of norm_groups")
+        elif kind == "mlstm":
+            mix = MixerSpec(kind, heads=int(m["heads"]), dim=int(m["dim"]), vdim=int(m["vdim"]),
+                            gate_cap=float(m["gate_cap"]))
+        else:
+            raise ValueError(f"unknown mixer type {kind!r}")
+        f = L.get("mlp")
+        mlp = None
+        if f:
+            if f["kind"] == "dense":
+                mlp = DenseSpec(int(f["ff"]), act="polynorm")
+            elif f["kind"] == "moe":
+                r = f["router"]
+                g = r.get("groups") or {}
+                mlp = MoESpec(int(r["experts"]), int(r["top"]), 1.0, int(f["expert"]["ff"]), act="swiglu", score="sigmoid",
+                              group_count=int(g.get("count", 1)), group_keep=int(g.get("keep", g.get("count", 1))))
+                if mlp.experts % mlp.group_count or not 1 <= mlp.group_keep <= mlp.group_count \
+                        or mlp.top > mlp.group_keep * (mlp.experts // mlp.group_count):
+                    raise ValueError("router: experts / groups / top do not fit")
+            else:
+                raise ValueError(f"unknown feed-forward kind {f['kind']!r}")
+        layers.append(LayerSpec(mix, mlp))
+    groups = int(raw["norm"].get("groups", 1))
+    if W % groups:
+        raise ValueError("width must be a multiple of norm.groups")
+    return HybridConfig(name, "pebodra", W, int(raw["vocab"]), tuple(layers), rms_eps=float(raw["norm"]["eps"]),
+                        norm_groups=groups, logit_softcap=float(raw.get("logit_softcap") or 0.0))
+
+
 # config.json "architecture" -> parser of that design's keys
-ARCHITECTURES = {"Filevik": filevik_config, "Sedopel": sedopel_config}
+ARCHITECTURES = {"Filevik": filevik_config, "Sedopel": sedopel_config, "Pebodra": pebodra_config}
 
 AnyConfig = Union[ModelConfig, HybridConfig]
 

@@ -1,6 +1,7 @@
-"""Layer-list decoders (Filevik, Sedopel): every layer has a token mixer (Mamba-1 selective scan,
-retention, latent attention, gated delta rule, or grouped-query softmax attention beside lightning
-attention) and an optional feed-forward (mixture of experts or dense), in the order config.json gives.
+"""Layer-list decoders (Filevik, Sedopel, Pebodra): every layer has a token mixer (Mamba-1 selective
+scan, retention, latent attention, gated delta rule, grouped-query softmax attention beside lightning
+attention, differential sliding-window attention, Mamba-2, mLSTM) and an optional feed-forward
+(mixture of experts or dense), in the order config.json gives.
 
 The residual stream lives in f32; each sublayer reads its rounding to the model dtype and adds
 ``rmsnorm(sublayer(x)) * w`` (ops.seqmix.norm_resadd: the f32 add, the norm and the rounded copy in
@@ -28,7 +29,19 @@ they do not take and for f32 models), everything between them on the HIP kernels
              out-proj.  Right: lightning attention (the retention kernels on SiLU'd inputs, heads
              normed together, sigmoid gate) -> out-proj.  The two outputs are normed and averaged
              in the launch that also adds the sublayer to the stream.
-  dense      up-proj -> erf GELU -> down-proj
+  dense      up-proj -> erf GELU or PolyNorm -> down-proj
+  diff_attn  one fused q | k | v projection -> biases, weighted RMS norm of every q / k map, rotation,
+             k and v to their pages (a layer with ``kv_from`` projects q alone and reads that layer's
+             pages) -> windowed causal softmax attention with the two maps of a head as two query
+             rows over the shared values (f32 out) -> a1 - lambda a2, unit RMS per head -> out-proj
+  mamba2     one fused projection (z | x | B | C | dt) -> causal conv + SiLU over x | B | C ->
+             recurrence with a scalar decay per head (f32 state per slot) -> y silu(z), RMS norm in
+             groups -> out-proj
+  mlstm      one fused projection (q | k | v | gate | input gate | forget gate) -> matrix memory with
+             a running maximum and a normaliser (f32 state per slot; unit-RMS heads, weight and
+             sigmoid gate in the kernel) -> out-proj
+  experts    (sigmoid scores) f32 router logits -> group-limited top-k, weights = scores -> grouped
+             SwiGLU expert GEMMs or their dense form
 
 Layer forms: ``x += norm(sublayer(x))`` (Filevik) or, with ``cfg.pre_norm``, a norm on both sides,
 ``x += norm_b(sublayer(norm(x)))``; with ``cfg.depth_average`` a layer hands on a learned weighted
@@ -125,6 +138,32 @@ class HybridModel:
                 t[p + "mix.right.v"], t[p + "mix.right.g"] = lin(b.heads * b.vdim, W), lin(b.heads * b.vdim, W)
                 t[p + "mix.right.o"], t[p + "mix.right.norm"] = lin(W, b.heads * b.vdim), torch.ones(b.heads * b.vdim)
                 t[p + "mix.left.out"], t[p + "mix.right.out"] = torch.ones(W), torch.ones(W)
+            elif m.kind == "diff_attention":
+                nq, nk = m.heads * 2 * m.dim, m.kv_heads * 2 * m.dim
+                t[p + "mix.q"], t[p + "mix.q.b"], t[p + "mix.q.norm"] = lin(nq, W), rnd(nq, s=0.1), torch.ones(m.dim)
+                if m.kv_from is None:
+                    t[p + "mix.k"], t[p + "mix.k.b"], t[p + "mix.k.norm"] = lin(nk, W), rnd(nk, s=0.1), torch.ones(m.dim)
+                    t[p + "mix.v"], t[p + "mix.v.b"] = lin(m.kv_heads * m.vdim, W), rnd(m.kv_heads * m.vdim, s=0.1)
+                for n_ in ("lq1", "lk1", "lq2", "lk2"):
+                    t[p + "mix." + n_] = rnd(m.dim, s=0.1)
+                t[p + "mix.o"], t[p + "mix.o.b"] = lin(W, m.heads * m.vdim), rnd(W, s=0.1)
+            elif m.kind == "mamba2":
+                inner, bc = m.heads * m.vdim, 2 * m.groups * m.state
+                t[p + "mix.in"] = lin(2 * inner + bc + m.heads, W)
+                t[p + "mix.conv"] = rnd(inner + bc, m.conv, s=1.0 / math.sqrt(m.conv))
+                t[p + "mix.conv.b"] = rnd(inner + bc, s=0.1)
+                dt = torch.exp(torch.rand(m.heads, generator=g) * (math.log(0.1) - math.log(0.001)) + math.log(0.001))
+                t[p + "mix.dt_bias"] = dt + torch.log(-torch.expm1(-dt))
+                t[p + "mix.A_log"] = torch.log(torch.rand(m.heads, generator=g) * 15 + 1)
+                t[p + "mix.D"], t[p + "mix.norm"] = torch.ones(m.heads), torch.ones(inner)
+                t[p + "mix.o"] = lin(W, inner)
+            elif m.kind == "mlstm":
+                hd, hv = m.heads * m.dim, m.heads * m.vdim
+                t[p + "mix.q"], t[p + "mix.k"], t[p + "mix.v"] = lin(hd, W), lin(hd, W), lin(hv, W)
+                t[p + "mix.g"], t[p + "mix.o"], t[p + "mix.norm"] = lin(hv, W), lin(W, hv), torch.ones(hv)
+                t[p + "mix.i"], t[p + "mix.f"] = lin(m.heads, W), lin(m.heads, W)
+                t[p + "mix.i.b"] = rnd(m.heads, s=0.1)
+                t[p + "mix.f.b"] = torch.linspace(3.0, 6.0, m.heads)
             elif m.kind == "mamba1":
                 t[p + "mix.in"] = lin(2 * m.inner, W)
                 t[p + "mix.conv"] = rnd(m.inner, m.conv, s=1.0 / math.sqrt(m.conv))
@@ -152,11 +191,15 @@ class HybridModel:
                 if cfg.pre_norm:
                     t[p + "norm2b"] = torch.ones(W)
                 t[p + "mlp.up"], t[p + "mlp.down"] = lin(f.ff, W), lin(W, f.ff)
+                if f.act == "polynorm":
+                    t[p + "mlp.act"] = torch.tensor([1.0, 0.5, 0.25, 0.0])
             elif f is not None:
                 t[p + "norm2"] = torch.ones(W)
                 t[p + "mlp.router"] = lin(f.experts, W)
                 for e in range(f.experts):
                     t[p + f"mlp.e{e}.up"], t[p + f"mlp.e{e}.down"] = lin(f.ff, W), lin(W, f.ff)
+                    if f.act == "swiglu":
+                        t[p + f"mlp.e{e}.gate"] = lin(f.ff, W)
                 if f.shared_ff:
                     t[p + "mlp.shared.up"], t[p + "mlp.shared.down"] = lin(f.shared_ff, W), lin(W, f.shared_ff)
         return t
@@ -211,6 +254,33 @@ class HybridModel:
                 D["lout"], D["rout"] = f32(t[p + "mix.left.out"]), f32(t[p + "mix.right.out"])
                 assert D["qscale"].numel() == a.heads and D["rnorm"].numel() == b.heads * b.vdim
                 assert D["proj"].shape[0] == self._left_cols(a) + 2 * b.heads * (b.dim + b.vdim)
+            elif m.kind == "diff_attention":
+                own = m.kv_from is None
+                names = ("q", "k", "v") if own else ("q",)
+                D["proj"] = put(torch.cat([t[p + "mix." + n] for n in names], 0))
+                D["bias"] = f32(torch.cat([t[p + f"mix.{n}.b"] for n in names], 0))
+                D["qnorm"] = f32(t[p + "mix.q.norm"])
+                D["knorm"] = f32(t[p + "mix.k.norm"]) if own else D["qnorm"]
+                l1 = (f32(t[p + "mix.lq1"]) * f32(t[p + "mix.lk1"])).sum()
+                l2 = (f32(t[p + "mix.lq2"]) * f32(t[p + "mix.lk2"])).sum()
+                D["lam"] = float(torch.exp(l1) - torch.exp(l2)) + m.diff       # one number for the layer
+                D["o"], D["ob"] = put(t[p + "mix.o"]), f32(t[p + "mix.o.b"])
+                cols = 2 * m.heads * m.dim + ((2 * m.kv_heads * m.dim + m.kv_heads * m.vdim) if own else 0)
+                assert D["proj"].shape[0] == cols == D["bias"].numel() and D["qnorm"].numel() == m.dim
+                assert tuple(D["o"].shape) == (W, m.heads * m.vdim)
+            elif m.kind == "mamba2":
+                inner, bc = m.heads * m.vdim, 2 * m.groups * m.state
+                D["in"], D["o"] = put(t[p + "mix.in"]), put(t[p + "mix.o"])
+                D["conv"], D["conv_b"] = f32(t[p + "mix.conv"]), f32(t[p + "mix.conv.b"])
+                D["dt_b"], D["D"] = f32(t[p + "mix.dt_bias"]), f32(t[p + "mix.D"])
+                D["neg_a"], D["gnorm"] = -torch.exp(f32(t[p + "mix.A_log"])), f32(t[p + "mix.norm"])
+                assert D["in"].shape[0] == 2 * inner + bc + m.heads and tuple(D["conv"].shape) == (inner + bc, m.conv)
+                assert D["neg_a"].numel() == m.heads and D["gnorm"].numel() == inner
+            elif m.kind == "mlstm":
+                D["proj"] = put(torch.cat([t[p + "mix." + n] for n in ("q", "k", "v", "g", "i", "f")], 0))
+                D["gate_b"] = f32(torch.cat([t[p + "mix.i.b"], t[p + "mix.f.b"]], 0))
+                D["hnorm"], D["o"] = f32(t[p + "mix.norm"]), put(t[p + "mix.o"])
+                assert D["proj"].shape[0] == 2 * m.heads * (m.dim + m.vdim + 1) and D["hnorm"].numel() == m.heads * m.vdim
             elif m.kind == "mamba1":
                 D["in"], D["x"], D["dt"], D["o"] = (put(t[p + "mix." + n]) for n in ("in", "x", "dt", "o"))
                 D["conv"], D["conv_b"] = f32(t[p + "mix.conv"]), f32(t[p + "mix.conv.b"])
@@ -234,10 +304,19 @@ class HybridModel:
                 if cfg.pre_norm:
                     D["norm2b"] = f32(t[p + "norm2b"])
                 assert tuple(D["up"].shape) == (f.ff, W)
+                if f.act == "polynorm":
+                    D["act"] = f32(t[p + "mlp.act"])
+                    assert D["act"].numel() == 4
             elif f is not None:
                 D["norm2"] = f32(t[p + "norm2"])
                 D["router"] = put(t[p + "mlp.router"])
-                w1 = torch.stack([t[p + f"mlp.e{e}.up"] for e in range(f.experts)])       # [E, ff, W]
+                if f.score == "sigmoid":
+                    D["router"] = f32(t[p + "mlp.router"])     # the router runs in f32
+                if f.act == "swiglu":      # per expert: gate rows, then up rows
+                    w1 = torch.stack([torch.cat([t[p + f"mlp.e{e}.gate"], t[p + f"mlp.e{e}.up"]], 0)
+                                      for e in range(f.experts)])                         # [E, 2 ff, W]
+                else:
+                    w1 = torch.stack([t[p + f"mlp.e{e}.up"] for e in range(f.experts)])   # [E, ff, W]
                 w2 = torch.stack([t[p + f"mlp.e{e}.down"] for e in range(f.experts)])     # [E, W, ff]
                 D["w1"] = put(w1)
                 grouped = (dt == torch.bfloat16 and dev.type == "cuda" and W % 32 == 0 and f.ff % 32 == 0
@@ -252,13 +331,15 @@ class HybridModel:
 
     def weight_bytes(self) -> int:
         n = sum(x.numel() * x.element_size() for x in (self.embed, self.lm_head, self.final_norm))
-        return n + sum(x.numel() * x.element_size() for L in self.layers for x in L.values())
+        return n + sum(x.numel() * x.element_size() for L in self.layers for x in L.values() if torch.is_tensor(x))
 
     def decode_read_bytes(self, top_only: bool = True) -> int:
         """Weight bytes one decode token reads (routed experts: ``top`` of them)."""
         n = self.lm_head.numel() * self.lm_head.element_size()
         for L, S in zip(self.layers, self.cfg.layers):
             for k, x in L.items():
+                if not torch.is_tensor(x):
+                    continue
                 b = x.numel() * x.element_size()
                 if k in ("w1", "w2", "w2d") and top_only and isinstance(S.mlp, MoESpec):
                     b = b * S.mlp.top // S.mlp.experts
@@ -290,6 +371,8 @@ class HybridModel:
                     n += block_size * (m.kv_rank + m.rot_dim) * it
                 elif m.kind == "softmax_attention":
                     n += block_size * m.kv_heads * (m.dim + m.vdim) * it
+                elif m.kind == "diff_attention" and m.kv_from is None:
+                    n += block_size * m.kv_heads * (2 * m.dim + m.vdim) * it
         return n
 
     def alloc_caches(self, num_blocks: int, block_size: int, slots: int) -> List[tuple]:
@@ -298,11 +381,29 @@ class HybridModel:
         (retention state [slots, heads, dim, vdim] f32,) / delta: (conv inputs [slots, taps - 1,
         q | k | v channels], state [slots, heads, vdim, dim] f32) / parallel: (paged keys [blocks,
         kv_heads, block, dim], paged values [blocks, kv_heads, vdim, block], lightning state [slots,
-        heads, dim, vdim] f32)."""
+        heads, dim, vdim] f32) / diff_attention: (paged keys [blocks, 2 kv_heads, block, dim], paged
+        values [blocks, kv_heads, vdim, block]), for a layer with ``kv_from`` the tensors of that
+        layer / mamba2: (conv inputs [slots, taps - 1, x | B | C channels], state [slots, heads, N,
+        vdim] f32) / mlstm: (memory [slots, heads, dim, vdim] f32, normaliser and maximum [slots,
+        heads, column blocks, dim + 1] f32)."""
         dev, out = self.device, []
         for L in self.cfg.layers:
             m = L.mixer
-            if m.kind == "delta":
+            if m.kind == "diff_attention":
+                if m.kv_from is not None:
+                    out.append(out[m.kv_from])
+                else:
+                    out.append((torch.zeros((num_blocks, 2 * m.kv_heads, block_size, m.dim), dtype=self.dtype, device=dev),
+                                torch.zeros((num_blocks, m.kv_heads, m.vdim, block_size), dtype=self.dtype, device=dev)))
+            elif m.kind == "mamba2":
+                c = m.heads * m.vdim + 2 * m.groups * m.state
+                out.append((torch.zeros((slots, max(m.conv - 1, 0), c), dtype=self.dtype, device=dev),
+                            torch.zeros((slots, m.heads, m.state, m.vdim), dtype=torch.float32, device=dev)))
+            elif m.kind == "mlstm":
+                out.append((torch.zeros((slots, m.heads, m.dim, m.vdim), dtype=torch.float32, device=dev),
+                            torch.zeros((slots, m.heads, seqmix.scan_col_blocks(m.vdim), m.dim + 1), dtype=torch.float32,
+                                        device=dev)))
+            elif m.kind == "delta":
                 c = 2 * m.kv_heads * m.dim + m.heads * m.vdim
                 out.append((torch.zeros((slots, max(m.conv - 1, 0), c), dtype=self.dtype, device=dev),
                             torch.zeros((slots, m.heads, m.vdim, m.dim), dtype=torch.float32, device=dev)))
@@ -402,10 +503,72 @@ class HybridModel:
                                         meta.qstart, meta.qlen, meta.ctx, meta.state_rows)
         return _mm(lo, L["lo"]), _mm(ro, L["ro"])
 
+    def _diff_attention(self, L, m: MixerSpec, x, positions, meta, cache):
+        """Both maps of every head run as rows of one grouped-query attention over 2 kv_heads key
+        heads and kv_heads shared value heads; the maps are combined afterwards."""
+        k_cache, v_cache = cache
+        own = m.kv_from is None
+        proj = _mm(x, L["proj"])
+        rot = m.rot.dims if m.rot is not None else 0
+        table = self._table(m) if rot else self._any_table()
+        q = seqmix.qk_norm_prep(proj, L["bias"], m.heads, m.kv_heads, 2, m.dim, m.vdim, L["qnorm"], L["knorm"], table, rot,
+                                self.cfg.rms_eps, m.scale, positions, meta.slots, k_cache if own else None,
+                                v_cache if own else None)
+        H2, G2 = 2 * m.heads, 2 * m.kv_heads
+        mfma = seqmix.gqa_use_mfma(q, H2, G2, m.dim, m.vdim, k_cache.shape[2])
+        ts, tt = meta.latent_tiles(1, self.device, seqmix.gqa_tokens_per_tile(H2, G2, mfma))
+        splits = seqmix.gqa_splits(int(ts.numel()), G2, meta.max_ctx, m.window) if mfma else 1
+        a = seqmix.paged_gqa_attention(q, k_cache, v_cache, meta.block_tables, meta.qstart, meta.qlen, meta.ctx, ts, tt,
+                                       None, mfma, splits, window=m.window, out_f32=True)
+        o = seqmix.diff_combine(a, m.heads, m.kv_heads, m.vdim, L["lam"], self.cfg.rms_eps, 1.0 - m.diff, self.dtype)
+        return _mm(o, L["o"])
+
+    def _mamba2(self, L, m: MixerSpec, x, meta, cache):
+        conv_state, state = cache
+        rows = meta.state_rows
+        inner = m.heads * m.vdim
+        proj = _mm(x, L["in"])                                          # z | x | B | C | dt
+        xbc_in = proj[:, inner:]
+        single = meta.host_qlen is None      # a decode step: the convolution refills its slots itself
+        xbc = seqmix.causal_conv_silu(xbc_in, L["conv"], L["conv_b"], conv_state, meta.qstart, meta.qlen, meta.ctx, rows,
+                                      refill=single)
+        if not single:
+            seqmix.conv_state_refill(xbc_in, conv_state, meta.qstart, meta.qlen, meta.ctx, rows)
+        y = seqmix.ssd_scan(xbc, proj, 2 * inner + 2 * m.groups * m.state, m.heads, m.vdim, m.state, m.groups, L["dt_b"],
+                            L["neg_a"], L["D"], state, meta.qstart, meta.qlen, meta.ctx, rows)
+        return _mm(seqmix.gated_group_norm(y, proj, L["gnorm"], m.norm_groups, self.cfg.rms_eps, self.dtype), L["o"])
+
+    def _mlstm(self, L, m: MixerSpec, x, meta, cache):
+        state, nm = cache
+        proj = _mm(x, L["proj"])                                        # q | k | v | gate | input gate | forget gate
+        o = seqmix.mlstm(proj, m.heads, m.dim, m.vdim, L["gate_b"], m.gate_cap, state, nm, self.cfg.rms_eps, L["hnorm"],
+                         meta.qstart, meta.qlen, meta.ctx, meta.state_rows)
+        return _mm(o, L["o"])
+
     def _dense(self, L, f: DenseSpec, x):
-        return _mm(seqmix.gelu_erf(_mm(x, L["up"])), L["down"])
+        z = _mm(x, L["up"])
+        a = seqmix.polynorm(z, L["act"], self.cfg.rms_eps) if f.act == "polynorm" else seqmix.gelu_erf(z)
+        return _mm(a, L["down"])
+
+    def _experts_swiglu(self, L, f: MoESpec, x):
+        """Sigmoid router in f32 with group-limited top-k, weights = the chosen scores; SwiGLU experts
+        on the grouped MFMA kernels, or in the dense form (all experts' columns in two GEMMs, unused
+        experts gated to zero) for f32 models and widths the grouped kernels do not take."""
+        logits = F.linear(x.float(), L["router"])
+        ids, w = seqmix.group_router(logits, f.top, f.group_count, f.group_keep)
+        if f.scale != 1.0:
+            w = w * f.scale
+        if "w2" in L and (not x.is_cuda or seqmix.moe_ffn_relu2_ok(x, L["w1"])):
+            return ops.moe_ffn(x, ids, w, L["w1"], L["w2"])
+        if "w2d" not in L:
+            L["w2d"] = L["w2"].permute(1, 0, 2).reshape(x.shape[1], -1).contiguous()
+        g = seqmix.dense_gate(ids, w, f.experts)
+        a = seqmix.swiglu_scale(_mm(x, L["w1"].view(f.experts * 2 * f.ff, -1)), g, f.ff)
+        return _mm(a, L["w2d"])
 
     def _experts(self, L, f: MoESpec, x):
+        if f.act == "swiglu":
+            return self._experts_swiglu(L, f, x)
         if f.experts > 64 or f.top > 8:      # beyond the router kernels' register budget: library top-k
             val, ids = torch.topk(torch.softmax(F.linear(x.float(), L["router"].float()), -1), f.top, -1)
             ids, w = ids.to(torch.int32), val / (val.sum(-1, keepdim=True) + 1e-20)
@@ -467,6 +630,12 @@ class HybridModel:
                 y = self._delta(L, m, h, meta, cache)
             elif m.kind == "parallel":
                 y = self._parallel(L, m, h, positions, meta, cache)
+            elif m.kind == "diff_attention":
+                y = self._diff_attention(L, m, h, positions, meta, cache)
+            elif m.kind == "mamba2":
+                y = self._mamba2(L, m, h, meta, cache)
+            elif m.kind == "mlstm":
+                y = self._mlstm(L, m, h, meta, cache)
             else:
                 y = self._latent(L, m, h, positions, meta, cache)
             if cfg.pre_norm:
@@ -488,10 +657,12 @@ class HybridModel:
                     h = torch.empty((T, W), dtype=self.dtype, device=x.device)
                     seqmix.resadd_norm(a, post, eps, x, nxt, h, **pair)
             else:
-                seqmix.norm_resadd(y, L["norm1"], eps, x, xl)
+                ng = cfg.norm_groups
+                seqmix.norm_resadd(y, L["norm1"], eps, x, xl, groups=ng, bias=L.get("ob"))
                 if S.mlp is not None:
-                    y = self._experts(L, S.mlp, x if xl is None else xl)
-                    seqmix.norm_resadd(y, L["norm2"], eps, x, xl)
+                    hin = x if xl is None else xl
+                    y = self._dense(L, S.mlp, hin) if isinstance(S.mlp, DenseSpec) else self._experts(L, S.mlp, hin)
+                    seqmix.norm_resadd(y, L["norm2"], eps, x, xl, groups=ng)
                 if X is not None:
                     x = seqmix.depth_mix(X, L["dwa"], i + 2)
                     if xl is not None:
@@ -501,14 +672,19 @@ class HybridModel:
         if cfg.pre_norm:     # h is the final-normed stream of every row
             return h if meta.all_last else h.index_select(0, meta.last_idx)
         sel = x if meta.all_last else x.index_select(0, meta.last_idx)
-        return seqmix.rms_rows(sel, self.final_norm, eps, out_dtype=self.dtype)
+        return seqmix.rms_rows(sel, self.final_norm, eps, out_dtype=self.dtype, groups=cfg.norm_groups)
 
     def logits(self, hidden: torch.Tensor) -> torch.Tensor:
         lg = _mm(hidden, self.lm_head)
+        if self.cfg.logit_softcap > 0:
+            return seqmix.softcap(lg, self.cfg.logit_softcap).to(lg.dtype)
         return lg if self.cfg.logit_scale == 1.0 else lg * self.cfg.logit_scale
 
     def logits_f32(self, hidden: torch.Tensor) -> torch.Tensor:
-        return _mm(hidden, self.lm_head).float() * self.cfg.logit_scale
+        lg = _mm(hidden, self.lm_head)
+        if self.cfg.logit_softcap > 0:
+            return seqmix.softcap(lg, self.cfg.logit_softcap)
+        return lg.float() * self.cfg.logit_scale
 
     def _sampler_logits(self, hidden: torch.Tensor) -> torch.Tensor:
         """bf16 logits [S, vocab] whose rows start 16-byte aligned (the sampler kernels read vectors)."""

@@ -375,17 +375,20 @@ def _seq_meta(qstart, qlen, ctx, rows):
     return [(qs[i], ql[i], cx[i], rw[i]) for i in range(len(qs)) if ql[i] > 0]
 
 
-def rms_rows(x, w, eps, out_dtype=None):
+def rms_rows(x, w, eps, out_dtype=None, groups=1):
+    """``groups`` > 1: each of that many equal consecutive parts of a row by its own root mean square."""
     xf = x.float()
-    y = xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + eps)
+    if groups > 1:
+        xf = xf.reshape(*x.shape[:-1], groups, x.shape[-1] // groups)
+    y = (xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + eps)).reshape(x.shape)
     if w is not None:
         y = y * w.float()
     return y.to(out_dtype or x.dtype)
 
 
-def norm_resadd(y, w, eps, x, x_lp=None):
-    """x (f32 residual stream, in place) += rmsnorm(y) * w; ``x_lp`` receives x rounded to its dtype."""
-    x += rms_rows(y, w, eps, torch.float32)
+def norm_resadd(y, w, eps, x, x_lp=None, groups=1, bias=None):
+    """x (f32 residual stream, in place) += rmsnorm(y (+ bias)) * w; ``x_lp`` receives x rounded to its dtype."""
+    x += rms_rows(y if bias is None else y.float() + bias.float(), w, eps, torch.float32, groups)
     if x_lp is not None:
         x_lp.copy_(x)
     return x
@@ -608,13 +611,16 @@ def attn_prep(proj, heads, kv_heads, dim, vdim, cos_sin, rot_dims, eps, qscale, 
     return q.to(proj.dtype)
 
 
-def paged_gqa_attention(q, k_cache, v_cache, block_tables, qstart, qlen, ctx, gate=None):
+def paged_gqa_attention(q, k_cache, v_cache, block_tables, qstart, qlen, ctx, gate=None, window=0, out_f32=False):
     """Causal softmax attention of q [T, heads, dim] (already scaled) over paged keys / values;
-    query head h reads key/value head h // (heads / kv_heads); the output [T, heads * vdim] is
-    multiplied by sigmoid(gate) when a gate [T, heads * vdim] is given."""
+    query head h reads key head h // (heads / kv_heads); the output [T, heads * vdim] is
+    multiplied by sigmoid(gate) when a gate [T, heads * vdim] is given.  ``window`` > 0: position i
+    sees keys i - window < j <= i.  A value cache with fewer heads than the key cache is shared by
+    neighbouring key heads (key head g reads value head g // (key heads / value heads))."""
     T, H, d = q.shape
     G, BSz, dv = k_cache.shape[1], k_cache.shape[2], v_cache.shape[2]
-    out = torch.zeros((T, H * dv), dtype=q.dtype, device=q.device)
+    vrep = G // v_cache.shape[1]
+    out = torch.zeros((T, H * dv), dtype=torch.float32 if out_f32 else q.dtype, device=q.device)
     qs, ql, cx = qstart.tolist(), qlen.tolist(), ctx.tolist()
     for s in range(len(qs)):
         n, c = ql[s], cx[s]
@@ -623,16 +629,19 @@ def paged_gqa_attention(q, k_cache, v_cache, block_tables, qstart, qlen, ctx, ga
         nb = (c + BSz - 1) // BSz
         blocks = block_tables[s, :nb].long()
         K = k_cache[blocks].transpose(1, 2).reshape(nb * BSz, G, d)[:c].float().repeat_interleave(H // G, 1)
-        V = v_cache[blocks].permute(0, 3, 1, 2).reshape(nb * BSz, G, dv)[:c].float().repeat_interleave(H // G, 1)
+        V = v_cache[blocks].permute(0, 3, 1, 2).reshape(nb * BSz, G // vrep, dv)[:c].float().repeat_interleave(
+            vrep * (H // G), 1)
         qq = q[qs[s]:qs[s] + n].float()
         sc = torch.einsum("thd,uhd->htu", qq, K)
         pos = torch.arange(c - n, c, device=q.device)
         mask = torch.arange(c, device=q.device)[None, :] > pos[:, None]
+        if window > 0:
+            mask = mask | (torch.arange(c, device=q.device)[None, :] <= pos[:, None] - window)
         sc = sc.masked_fill(mask[None], float("-inf"))
         o = torch.einsum("htu,uhv->thv", torch.softmax(sc, -1), V).reshape(n, H * dv)
         if gate is not None:
             o = o * torch.sigmoid(gate[qs[s]:qs[s] + n].float())
-        out[qs[s]:qs[s] + n] = o.to(q.dtype)
+        out[qs[s]:qs[s] + n] = o.to(out.dtype)
     return out
 
 
@@ -705,3 +714,171 @@ def delta_rule(qkv, gba, heads, kv_heads, dim, vdim, neg_a, dt_bias, norm_w, eps
         o = o * torch.rsqrt(o.pow(2).mean(-1, keepdim=True) + eps) * norm_w.float()[None, None, :]
         out[q0:q0 + n] = (o.reshape(n, H * dv) * torch.nn.functional.silu(gate)).to(qkv.dtype)
     return out
+
+
+# ----------------------------------------------------------------------------- differential attention
+
+def qk_norm_prep(proj, bias, heads, kv_heads, maps, dim, vdim, qnorm_w, knorm_w, cos_sin, rot_dims, eps, qscale,
+                 positions, slots, k_cache, v_cache):
+    """proj [T, >= heads maps dim (+ kv_heads maps dim + kv_heads vdim)] (q | k | v) plus ``bias``
+    (f32, same columns).  Every (head, map) vector of q and k: RMS norm over ``dim`` times the shared
+    weight, then rotate-half positions on its first ``rot_dims`` dims; q times ``qscale``.  q comes
+    back as [T, heads maps, dim] with the heads of a key/value head ordered (map, head in group), so
+    that query row r reads key row r // (heads / kv_heads) of k_cache [blocks, kv_heads maps, block,
+    dim]; v goes to v_cache [blocks, kv_heads, vdim, block].  Without caches (a layer that reads
+    another layer's) only q is made."""
+    T, H, G, M, d, dv = proj.shape[0], heads, kv_heads, maps, dim, vdim
+    nq, nk = H * M * d, G * M * d
+    pf = proj.float()
+    if bias is not None:
+        pf = pf[:, :bias.numel()] + bias.float()[None, :]
+    half = rot_dims // 2
+    c, s = _rot_table(cos_sin, positions, half) if half > 0 else (None, None)
+
+    def norm_rot(t, w):
+        t = t * torch.rsqrt(t.pow(2).mean(-1, keepdim=True) + eps) * w.float()
+        if half > 0:
+            u, w_ = t[..., :half].clone(), t[..., half:2 * half].clone()
+            t[..., :half] = u * c[:, None, :] - w_ * s[:, None, :]
+            t[..., half:2 * half] = w_ * c[:, None, :] + u * s[:, None, :]
+        return t
+
+    q = norm_rot(pf[:, :nq].reshape(T, H * M, d).clone(), qnorm_w) * qscale
+    q = q.view(T, G, H // G, M, d).transpose(2, 3).reshape(T, H * M, d)
+    if k_cache is not None:
+        k = norm_rot(pf[:, nq:nq + nk].reshape(T, G * M, d).clone(), knorm_w)
+        v = pf[:, nq + nk:nq + nk + G * dv].reshape(T, G, dv)
+        live = slots >= 0
+        sl = slots[live].long()
+        BSz = k_cache.shape[2]
+        k_cache[sl // BSz, :, sl % BSz] = k[live].to(k_cache.dtype)
+        v_cache[sl // BSz, :, :, sl % BSz] = v[live].to(v_cache.dtype)
+    return q.to(proj.dtype)
+
+
+def diff_combine(a, heads, kv_heads, vdim, lam, eps, out_scale, out_dtype):
+    """a [T, 2 heads vdim] f32: per key/value head the first-map outputs of its query heads, then the
+    second-map outputs.  o = a1 - lam a2 per head, to unit RMS over vdim, times ``out_scale``."""
+    T, R = a.shape[0], heads // kv_heads
+    a = a.float().view(T, kv_heads, 2, R, vdim)
+    o = (a[:, :, 0] - lam * a[:, :, 1]).reshape(T, heads, vdim)
+    o = o * torch.rsqrt(o.pow(2).mean(-1, keepdim=True) + eps) * out_scale
+    return o.reshape(T, heads * vdim).to(out_dtype)
+
+
+# ----------------------------------------------------------------------------- gated outer-product recurrences
+
+def ssd_scan(xbc, proj, dt_col, heads, vdim, n_state, groups, dt_bias, neg_a, D, state, qstart, qlen, ctx, rows):
+    """Mamba-2 recurrence.  xbc [T, heads vdim + 2 groups N] (x | B | C, convolved and activated),
+    step logits in proj[:, dt_col : dt_col + heads].  dt = softplus(. + dt_bias); per head (B, C of
+    group head // (heads / groups)):  S <- exp(neg_a dt) S + dt B x^T,  y = S^T C + D x.  state
+    [slots, heads, N, vdim] f32; returns y [T, heads vdim] f32."""
+    T, H, dv, N, G = xbc.shape[0], heads, vdim, n_state, groups
+    out = torch.zeros((T, H * dv), dtype=torch.float32, device=xbc.device)
+    rep = H // G
+    for q0, n, cx, row in _seq_meta(qstart, qlen, ctx, rows):
+        blk = xbc[q0:q0 + n].float()
+        x = blk[:, :H * dv].reshape(n, H, dv)
+        B = blk[:, H * dv:H * dv + G * N].reshape(n, G, N).repeat_interleave(rep, 1)
+        C = blk[:, H * dv + G * N:H * dv + 2 * G * N].reshape(n, G, N).repeat_interleave(rep, 1)
+        dt = torch.nn.functional.softplus(proj[q0:q0 + n, dt_col:dt_col + H].float() + dt_bias.float()[None, :])
+        dA = torch.exp(neg_a.float()[None, :] * dt)
+        S = state[row].clone() if cx - n > 0 else torch.zeros((H, N, dv), dtype=torch.float32, device=xbc.device)
+        y = torch.empty((n, H, dv), dtype=torch.float32, device=xbc.device)
+        for t in range(n):
+            S = dA[t][:, None, None] * S + (dt[t][:, None] * B[t])[:, :, None] * x[t][:, None, :]
+            y[t] = torch.einsum("hnv,hn->hv", S, C[t]) + D.float()[:, None] * x[t]
+        state[row] = S
+        out[q0:q0 + n] = y.reshape(n, H * dv)
+    return out
+
+
+def gated_group_norm(y, z, w, groups, eps, out_dtype):
+    """rmsnorm over each of ``groups`` equal parts of y silu(z), times w (y f32 [T, n], z [T, >= n])."""
+    g = y.float() * torch.nn.functional.silu(z[:, :y.shape[1]].float())
+    return rms_rows(g, w, eps, out_dtype, groups)
+
+
+def mlstm(proj, heads, dim, vdim, gate_b, cap, state, nm, eps, norm_w, qstart, qlen, ctx, rows):
+    """Matrix-memory LSTM.  proj [T, 2 heads dim + 2 heads vdim + 2 heads] (q | k | v | output gate |
+    input-gate logits | forget-gate logits), gate_b f32 [2 heads].  q times dim^-1/2;
+    i = cap tanh(. / cap), f = logsigmoid(cap tanh(. / cap)); with a running maximum m (0 at the
+    start):  m' = max(f + m, i),  S <- exp(f + m - m') S + exp(i - m') k v^T,  n likewise with k,
+    o = S^T q / (max(|n . q|, exp(-m')) + 1e-6).  Each head's o to unit RMS, times norm_w, times
+    sigmoid(gate).  state [slots, heads, dim, vdim] f32; nm [slots, heads, copies, dim + 1] f32
+    holds n and, last, m (every copy the same: the kernel keeps one per block of value columns)."""
+    T, H, d, dv = proj.shape[0], heads, dim, vdim
+    out = torch.zeros((T, H * dv), dtype=proj.dtype, device=proj.device)
+    logsig = torch.nn.functional.logsigmoid
+    for q0, n_, cx, row in _seq_meta(qstart, qlen, ctx, rows):
+        blk = proj[q0:q0 + n_].float()
+        q = blk[:, :H * d].reshape(n_, H, d) * (d ** -0.5)
+        k = blk[:, H * d:2 * H * d].reshape(n_, H, d)
+        v = blk[:, 2 * H * d:2 * H * d + H * dv].reshape(n_, H, dv)
+        g = blk[:, 2 * H * d + H * dv:2 * H * d + 2 * H * dv]
+        z = blk[:, 2 * H * d + 2 * H * dv:2 * H * d + 2 * H * dv + 2 * H] + gate_b.float()[None, :]
+        ig = cap * torch.tanh(z[:, :H] / cap)
+        fg = logsig(cap * torch.tanh(z[:, H:] / cap))
+        if cx - n_ > 0:
+            S, nv, m = state[row].clone(), nm[row, :, 0, :d].clone(), nm[row, :, 0, d].clone()
+        else:
+            S = torch.zeros((H, d, dv), dtype=torch.float32, device=proj.device)
+            nv, m = torch.zeros((H, d), dtype=torch.float32, device=proj.device), torch.zeros(H, device=proj.device)
+        o = torch.empty((n_, H, dv), dtype=torch.float32, device=proj.device)
+        for t in range(n_):
+            m2 = torch.maximum(fg[t] + m, ig[t])
+            a, b = torch.exp(fg[t] + m - m2), torch.exp(ig[t] - m2)
+            S = a[:, None, None] * S + b[:, None, None] * k[t][:, :, None] * v[t][:, None, :]
+            nv = a[:, None] * nv + b[:, None] * k[t]
+            m = m2
+            den = torch.maximum((nv * q[t]).sum(-1).abs(), torch.exp(-m)) + 1e-6
+            o[t] = torch.einsum("hdv,hd->hv", S, q[t]) / den[:, None]
+        state[row] = S
+        nm[row, :, :, :d] = nv[:, None, :]
+        nm[row, :, :, d] = m[:, None]
+        o = o * torch.rsqrt(o.pow(2).mean(-1, keepdim=True) + eps)
+        out[q0:q0 + n_] = (o.reshape(n_, H * dv) * norm_w.float()[None, :] * torch.sigmoid(g)).to(proj.dtype)
+    return out
+
+
+# ----------------------------------------------------------------------------- PolyNorm, grouped sigmoid router, SwiGLU experts
+
+def polynorm(z, coef, eps):
+    """a N(z) + b N(z^2) + c N(z^3) + e per row, N(u) = u / sqrt(mean(u^2) + eps); coef = (a, b, c, e) f32."""
+    zf = z.float()
+    a, b, c, e = coef.float().tolist()
+    N = lambda u: u * torch.rsqrt(u.pow(2).mean(-1, keepdim=True) + eps)
+    return (a * N(zf) + b * N(zf * zf) + c * N(zf * zf * zf) + e).to(z.dtype)
+
+
+def group_router(logits, top, count, keep):
+    """Scores = sigmoid(logits) [T, E] f32.  The experts form ``count`` groups of neighbours; a group
+    scores the sum of its two best experts; the ``top`` best experts inside the ``keep`` best groups
+    are chosen (ties: the lower index), weights = their scores.  -> ids [T, top] int32, w [T, top] f32."""
+    s = torch.sigmoid(logits.float())
+    T, E = s.shape
+    per = E // count
+    allowed = torch.ones((T, E), dtype=torch.bool, device=s.device)
+    if count > 1 and keep < count:
+        gs = s.view(T, count, per).topk(min(2, per), -1).values.sum(-1)
+        order = torch.sort(gs, dim=-1, descending=True, stable=True).indices[:, :keep]
+        ok = torch.zeros((T, count), dtype=torch.bool, device=s.device)
+        ok.scatter_(1, order, True)
+        allowed = ok.repeat_interleave(per, 1)
+    masked = torch.where(allowed, s, torch.full_like(s, -1.0))
+    ids = torch.sort(masked, dim=-1, descending=True, stable=True).indices[:, :top]
+    return ids.to(torch.int32), s.gather(1, ids)
+
+
+def swiglu_scale(gu, gate, ff):
+    """Dense form of routed SwiGLU experts: gu [T, E 2 ff] (per expert: gate columns, then up columns)
+    -> [T, E ff] = silu(gate part) * up part * gate[t, expert] (zero for experts the token does not use)."""
+    T = gu.shape[0]
+    g = gu.float().view(T, -1, 2, ff)
+    y = torch.nn.functional.silu(g[:, :, 0]) * g[:, :, 1] * gate.float()[:, :, None]
+    return y.reshape(T, -1).to(gu.dtype)
+
+
+def softcap(x, cap):
+    """cap * tanh(x / cap) in f32."""
+    return cap * torch.tanh(x.float() / cap)

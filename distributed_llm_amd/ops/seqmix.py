@@ -23,24 +23,26 @@ LAT_ROWS = 16      # (token, head) rows per workgroup of the latent attention ke
                    # (sequence, first token) covers max(1, 16 // heads) tokens (AttnMeta.latent_tiles)
 
 
-def rms_rows(x: torch.Tensor, w: Optional[torch.Tensor], eps: float, out_dtype=None) -> torch.Tensor:
-    """Row-wise x / sqrt(mean(x^2) + eps) (* w) for any row length; x may be a column slice."""
+def rms_rows(x: torch.Tensor, w: Optional[torch.Tensor], eps: float, out_dtype=None, groups: int = 1) -> torch.Tensor:
+    """Row-wise x / sqrt(mean(x^2) + eps) (* w) for any row length; x may be a column slice.
+    ``groups`` > 1: each of that many equal consecutive parts of a row by its own root mean square."""
     ext = _native(x)
     if ext is None:
-        return ref.rms_rows(x, w, eps, out_dtype)
+        return ref.rms_rows(x, w, eps, out_dtype, groups)
     y = torch.empty(x.shape, dtype=out_dtype or x.dtype, device=x.device)
-    ext.rms_rows(x, w, y, float(eps))
+    ext.rms_rows(x, w, y, float(eps), int(groups))
     return y
 
 
 def norm_resadd(y: torch.Tensor, w: torch.Tensor, eps: float, x: torch.Tensor,
-                x_lp: Optional[torch.Tensor] = None) -> torch.Tensor:
+                x_lp: Optional[torch.Tensor] = None, groups: int = 1, bias: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Residual update in f32: ``x += rmsnorm(y) * w`` in place (x f32 [T, H]); ``x_lp`` (the model
-    dtype) receives the rounded stream for the next projections, in the same launch."""
+    dtype) receives the rounded stream for the next projections, in the same launch.  ``groups`` as
+    in ``rms_rows``; ``bias`` (the sublayer's output bias) is added to y before the norm."""
     ext = _native(y)
     if ext is None:
-        return ref.norm_resadd(y, w, eps, x, x_lp)
-    ext.norm_resadd(y, w, float(eps), x, x_lp)
+        return ref.norm_resadd(y, w, eps, x, x_lp, groups, bias)
+    ext.norm_resadd(y, w, float(eps), x, x_lp, int(groups), bias)
     return x
 
 
@@ -278,32 +280,171 @@ GQA_SPLIT_TARGET = 512     # workgroups a small matrix-core attention grid is sp
 GQA_SPLIT_MAX = 16
 
 
-def gqa_splits(n_tiles: int, kv_heads: int, max_ctx: int) -> int:
+def gqa_splits(n_tiles: int, kv_heads: int, max_ctx: int, window: int = 0) -> int:
     """Key splits of a matrix-core attention launch: grids with few workgroups (decode steps at small
     batch, short portions) split every row's 64-key tiles over up to ``GQA_SPLIT_MAX`` workgroups."""
     tiles = (int(max_ctx) + 63) // 64 if max_ctx > 0 else GQA_SPLIT_MAX     # decode graphs: any context
+    if window > 0:
+        tiles = min(tiles, (int(window) + 62) // 64 + 1)
     return max(1, min(GQA_SPLIT_MAX, tiles, GQA_SPLIT_TARGET // max(1, n_tiles * kv_heads)))
 
 
 def paged_gqa_attention(q, k_cache, v_cache, block_tables, qstart, qlen, ctx, tile_seq, tile_tok0,
-                        gate: Optional[torch.Tensor] = None, mfma: bool = False, splits: int = 1) -> torch.Tensor:
+                        gate: Optional[torch.Tensor] = None, mfma: bool = False, splits: int = 1, window: int = 0,
+                        out_f32: bool = False) -> torch.Tensor:
     """Causal softmax attention over paged keys / values of any head widths (f32 scores, online
     softmax), output times sigmoid(gate).  ``tile_seq`` / ``tile_tok0``: one entry per
     ``gqa_tokens_per_tile(heads, kv_heads, mfma)`` new tokens of a sequence.  ``splits`` > 1
-    (matrix-core kernel): a row's keys are split over that many workgroups and merged."""
+    (matrix-core kernel): a row's keys are split over that many workgroups and merged.
+    ``window`` > 0: a position sees itself and the ``window - 1`` keys before it (older key tiles are
+    not read).  A value cache with fewer heads than the key cache is shared by neighbouring key
+    heads.  ``out_f32``: the output stays f32 whatever the model dtype."""
     ext = _native(q)
     if ext is None:
-        return ref.paged_gqa_attention(q, k_cache, v_cache, block_tables, qstart, qlen, ctx, gate)
+        return ref.paged_gqa_attention(q, k_cache, v_cache, block_tables, qstart, qlen, ctx, gate, window, out_f32)
     dv = v_cache.shape[2]
-    out = torch.zeros((q.shape[0], q.shape[1] * dv), dtype=q.dtype, device=q.device)
+    out = torch.zeros((q.shape[0], q.shape[1] * dv), dtype=torch.float32 if out_f32 else q.dtype, device=q.device)
     splits = int(splits) if mfma else 1
     part = None
     if splits > 1:
         part = torch.empty(int(tile_seq.numel()) * k_cache.shape[1] * splits * GQA_ROWS_MFMA * (dv + 2),
                            dtype=torch.float32, device=q.device)
     ext.paged_gqa_attention(q, k_cache, v_cache, block_tables, qstart, qlen, ctx, tile_seq, tile_tok0, gate, out,
-                            bool(mfma), splits, part)
+                            bool(mfma), splits, part, int(window))
     return out
+
+
+# ----------------------------------------------------------------------------- differential attention
+
+def qk_norm_prep(proj, bias, heads, kv_heads, maps, dim, vdim, qnorm_w, knorm_w, cos_sin, rot_dims, eps, qscale,
+                 positions, slots, k_cache, v_cache) -> torch.Tensor:
+    """Attention inputs with a weighted RMS norm of every q / k vector BEFORE its rotation, biases,
+    and ``maps`` score maps per head (differential attention: 2).  proj [T, q | k | v] (+ ``bias``
+    f32 over the same columns); returns q [T, heads maps, dim], scaled by ``qscale``, the query rows
+    of one key/value head ordered (map, head in group), so that the grouped-query kernels pair row r
+    with key row r // (heads / kv_heads) of k_cache [blocks, kv_heads maps, block, dim].  v goes to
+    v_cache [blocks, kv_heads, vdim, block].  ``k_cache`` None (a layer that reads another layer's
+    keys and values): proj holds q alone."""
+    ext = _native(proj)
+    if ext is None:
+        return ref.qk_norm_prep(proj, bias, heads, kv_heads, maps, dim, vdim, qnorm_w, knorm_w, cos_sin, rot_dims, eps,
+                                qscale, positions, slots, k_cache, v_cache)
+    q = torch.empty((proj.shape[0], heads * maps, dim), dtype=proj.dtype, device=proj.device)     # every row is written
+    ext.qk_norm_prep(proj, bias, int(heads), int(kv_heads), int(maps), int(dim), int(vdim), qnorm_w, knorm_w, cos_sin,
+                     int(rot_dims), float(eps), float(qscale), positions, slots, k_cache, v_cache, q)
+    return q
+
+
+def diff_combine(a, heads, kv_heads, vdim, lam, eps, out_scale, out_dtype) -> torch.Tensor:
+    """The two maps of differential attention into one output per head: a [T, 2 heads vdim] f32 in
+    the row order ``qk_norm_prep`` gives; o = a1 - lam a2, unit RMS over vdim, times ``out_scale``."""
+    ext = _native(a)
+    if ext is None:
+        return ref.diff_combine(a, heads, kv_heads, vdim, lam, eps, out_scale, out_dtype)
+    out = torch.empty((a.shape[0], heads * vdim), dtype=out_dtype, device=a.device)
+    ext.diff_combine(a, int(heads), int(kv_heads), int(vdim), float(lam), float(eps), float(out_scale), out)
+    return out
+
+
+# ----------------------------------------------------------------------------- gated outer-product recurrences (Mamba-2, mLSTM)
+
+SCAN_COLS = 32      # value columns of one (sequence, head) a workgroup of the recurrence kernels owns
+
+
+def scan_col_blocks(vdim: int) -> int:
+    """Workgroups per (sequence, head) of ``ssd_scan`` / ``mlstm``; an mLSTM keeps one copy of its
+    normaliser state per block."""
+    return (int(vdim) + SCAN_COLS - 1) // SCAN_COLS
+
+
+def ssd_scan(xbc, proj, dt_col, heads, vdim, n_state, groups, dt_bias, neg_a, D, state, qstart, qlen, ctx,
+             rows) -> torch.Tensor:
+    """Mamba-2 recurrence (scalar decay per head, B / C per group of heads): xbc [T, x | B | C]
+    convolved and activated, step logits in proj[:, dt_col:dt_col + heads]; dt = softplus(. + bias),
+    S <- exp(neg_a dt) S + dt B x^T, y = S^T C + D x.  state [slots, heads, N, vdim] f32; returns y f32."""
+    ext = _native(xbc)
+    if ext is None:
+        return ref.ssd_scan(xbc, proj, dt_col, heads, vdim, n_state, groups, dt_bias, neg_a, D, state, qstart, qlen, ctx,
+                            rows)
+    out = torch.zeros((xbc.shape[0], heads * vdim), dtype=torch.float32, device=xbc.device)
+    ext.ssd_scan(xbc, proj, int(dt_col), int(heads), int(vdim), int(n_state), int(groups), dt_bias, neg_a, D, state,
+                 qstart, qlen, ctx, rows, out)
+    return out
+
+
+def gated_group_norm(y, z, w, groups, eps, out_dtype) -> torch.Tensor:
+    """rmsnorm over each of ``groups`` equal parts of ``y silu(z)``, times w: y f32 [T, n], z the first
+    n columns of a [T, >= n] activation; the gate comes before the norm."""
+    ext = _native(y)
+    if ext is None:
+        return ref.gated_group_norm(y, z, w, groups, eps, out_dtype)
+    out = torch.empty(y.shape, dtype=out_dtype, device=y.device)
+    ext.gated_group_norm(y, z, w, int(groups), float(eps), out)
+    return out
+
+
+def mlstm(proj, heads, dim, vdim, gate_b, cap, state, nm, eps, norm_w, qstart, qlen, ctx, rows) -> torch.Tensor:
+    """Matrix-memory LSTM over proj [T, q | k | v | output gate | input-gate logits | forget-gate
+    logits] (``gate_b``: the two gates' biases): capped exponential input gate, sigmoid forget gate in
+    log space, running maximum from 0, normaliser max(|n . q|, exp(-m)) + 1e-6; heads to unit RMS times
+    ``norm_w`` times sigmoid(gate).  state [slots, heads, dim, vdim] f32, nm [slots, heads,
+    scan_col_blocks(vdim), dim + 1] f32 (n and m)."""
+    ext = _native(proj)
+    if ext is None:
+        return ref.mlstm(proj, heads, dim, vdim, gate_b, cap, state, nm, eps, norm_w, qstart, qlen, ctx, rows)
+    T = proj.shape[0]
+    raw = torch.zeros((T, heads * vdim), dtype=torch.float32, device=proj.device)
+    out = torch.empty((T, heads * vdim), dtype=proj.dtype, device=proj.device)      # the finish kernel writes every row
+    ext.mlstm(proj, int(heads), int(dim), int(vdim), gate_b, float(cap), state, nm, float(eps), norm_w, qstart, qlen,
+              ctx, rows, raw, out)
+    return out
+
+
+# ----------------------------------------------------------------------------- PolyNorm, grouped sigmoid router, SwiGLU experts
+
+def polynorm(z: torch.Tensor, coef: torch.Tensor, eps: float) -> torch.Tensor:
+    """a N(z) + b N(z^2) + c N(z^3) + e per row with N the scaling to unit RMS; coef f32 (a, b, c, e)."""
+    ext = _native(z)
+    if ext is None:
+        return ref.polynorm(z, coef, eps)
+    y = torch.empty_like(z)
+    ext.polynorm(z, coef, float(eps), y)
+    return y
+
+
+def group_router(logits: torch.Tensor, top: int, count: int, keep: int) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Sigmoid scores of f32 router logits [T, E]; ``count`` groups of neighbouring experts, a group
+    scores the sum of its two best, the ``top`` best experts of the ``keep`` best groups are chosen;
+    weights = their scores, not renormalised.  -> ids [T, top] int32, weights [T, top] f32."""
+    ext = _native(logits)
+    if ext is None:
+        return ref.group_router(logits, top, count, keep)
+    T = logits.shape[0]
+    ids = torch.empty((T, top), dtype=torch.int32, device=logits.device)
+    w = torch.empty((T, top), dtype=torch.float32, device=logits.device)
+    ext.group_router(logits, int(top), int(count), int(keep), ids, w)
+    return ids, w
+
+
+def swiglu_scale(gu: torch.Tensor, gate: torch.Tensor, ff: int) -> torch.Tensor:
+    """Dense form of routed SwiGLU experts: gu [T, E 2 ff] (per expert its gate columns, then its up
+    columns) -> [T, E ff] = silu(gate) * up * gate[t, expert]."""
+    ext = _native(gu)
+    if ext is None:
+        return ref.swiglu_scale(gu, gate, ff)
+    y = torch.empty((gu.shape[0], gu.shape[1] // 2), dtype=gu.dtype, device=gu.device)
+    ext.swiglu_scale(gu, gate, int(ff), y)
+    return y
+
+
+def softcap(x: torch.Tensor, cap: float) -> torch.Tensor:
+    """cap * tanh(x / cap), f32 out."""
+    ext = _native(x)
+    if ext is None:
+        return ref.softcap(x, cap)
+    y = torch.empty(x.shape, dtype=torch.float32, device=x.device)
+    ext.softcap(x, float(cap), y)
+    return y
 
 
 # ----------------------------------------------------------------------------- lightning attention, gated delta rule
