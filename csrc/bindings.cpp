@@ -48,8 +48,21 @@ int dllm_skinny_gemm(const void*, long, const void*, void*, long, int, int, int,
 int dllm_moe_max_tiles(int, int);
 int dllm_moe_ffn(const void*, long, long, int, const int*, const float*, int, int, const void*, const void*, int, int*,
                  int*, void*, float*, void*, int, hipStream_t);
-int dllm_rms_rows(const void*, long, int, const float*, void*, long, int, int, int, float, hipStream_t);
-int dllm_norm_resadd(const void*, long, int, const float*, float*, void*, int, int, float, hipStream_t);
+int dllm_rms_rows(const void*, long, int, const float*, void*, long, int, int, int, float, int, hipStream_t);
+int dllm_norm_resadd(const void*, long, int, const float*, float*, void*, int, int, float, int, const float*, hipStream_t);
+int dllm_polynorm(const void*, long, int, const float*, void*, long, int, float, hipStream_t);
+int dllm_group_router(const float*, int, int, int, int, int, int*, float*, hipStream_t);
+int dllm_swiglu_scale(const void*, int, const float*, int, int, void*, long, hipStream_t);
+int dllm_softcap(const void*, int, float, float*, long, hipStream_t);
+int dllm_gated_group_norm(const float*, const void*, long, int, const float*, void*, int, int, int, float, hipStream_t);
+int dllm_outer_scan_cols();
+int dllm_ssd_scan(const void*, long, const void*, long, int, int, int, int, int, int, const float*, const float*, const float*,
+                  float*, const int*, const int*, const int*, const int*, int, float*, hipStream_t);
+int dllm_mlstm(const void*, long, int, int, int, int, const float*, float, float*, float*, int, float, const float*, const int*,
+               const int*, const int*, const int*, int, long, float*, void*, hipStream_t);
+int dllm_qk_norm_prep(const void*, long, int, const float*, int, int, int, int, int, const float*, const float*, const float*,
+                      int, int, float, float, const int*, const int*, void*, void*, void*, long, int, hipStream_t);
+int dllm_diff_combine(const float*, void*, int, long, int, int, int, float, float, float, hipStream_t);
 int dllm_conv_silu(const void*, long, int, const float*, const float*, void*, const int*, const int*, const int*,
                    const int*, void*, int, int, int, int, int, hipStream_t);
 int dllm_selective_scan(const void*, const void*, int, const float*, const float*, const void*, long, int, const float*,
@@ -77,7 +90,8 @@ int dllm_attn_prep(const void*, long, int, int, int, int, int, const float*, int
 int dllm_gqa_tile_tokens(int, int, int);
 int dllm_gqa_mfma_ok(int, int, int, int, int, int);
 int dllm_paged_gqa(const void*, const void*, const void*, int, const int*, int, int, const int*, const int*, const int*,
-                   const int*, const int*, int, const void*, long, void*, int, int, int, int, int, int, float*, hipStream_t);
+                   const int*, const int*, int, const void*, long, void*, int, int, int, int, int, int, float*, int, int, int,
+                   hipStream_t);
 int dllm_relu2_scale(const void*, int, const float*, int, int, void*, long, int, hipStream_t);
 int dllm_dense_gate(const int*, const float*, float*, long, int, int, hipStream_t);
 int dllm_latent_kv_write(const void*, long, int, int, int, const float*, float, const int*, const float*, int, const int*,
@@ -1325,7 +1339,7 @@ SeqMeta seq_meta(const torch::Tensor& qstart, const torch::Tensor& qlen, const t
   return {S, qstart.data_ptr<int>(), qlen.data_ptr<int>(), ctx.data_ptr<int>(), rows.data_ptr<int>()};
 }
 
-void rms_rows(torch::Tensor x, c10::optional<torch::Tensor> w, torch::Tensor y, double eps) {
+void rms_rows(torch::Tensor x, c10::optional<torch::Tensor> w, torch::Tensor y, double eps, int64_t groups) {
   const bool xf = act_f32(x, "x"), yf = act_f32(y, "y");
   check_rows2d(x, "x");
   check_rows2d(y, "y");
@@ -1336,12 +1350,14 @@ void rms_rows(torch::Tensor x, c10::optional<torch::Tensor> w, torch::Tensor y, 
     TORCH_CHECK(w->numel() == x.size(1), "w length");
     wp = w->data_ptr<float>();
   }
+  TORCH_CHECK(groups >= 1 && x.size(1) % groups == 0, "row length must be a multiple of groups");
   ok(dllm_rms_rows(x.data_ptr(), x.stride(0), xf, wp, y.data_ptr(), y.stride(0), yf, (int)x.size(0), (int)x.size(1),
-                   (float)eps, stream()),
+                   (float)eps, (int)groups, stream()),
      "rms_rows");
 }
 
-void norm_resadd(torch::Tensor y, torch::Tensor w, double eps, torch::Tensor x, c10::optional<torch::Tensor> xl) {
+void norm_resadd(torch::Tensor y, torch::Tensor w, double eps, torch::Tensor x, c10::optional<torch::Tensor> xl,
+                 int64_t groups, c10::optional<torch::Tensor> bias) {
   const bool f = act_f32(y, "y");
   check_rows2d(y, "y");
   check_f32(w, "w");
@@ -1353,8 +1369,15 @@ void norm_resadd(torch::Tensor y, torch::Tensor w, double eps, torch::Tensor x, 
                 "x_lp: contiguous, the dtype of y, the shape of x");
     lp = xl->data_ptr();
   }
+  TORCH_CHECK(groups >= 1 && x.size(1) % groups == 0 && x.is_contiguous(), "width must be a multiple of groups; x contiguous");
+  const float* bp = nullptr;
+  if (bias) {
+    check_f32(*bias, "bias");
+    TORCH_CHECK(bias->numel() == x.size(1), "bias length");
+    bp = bias->data_ptr<float>();
+  }
   ok(dllm_norm_resadd(y.data_ptr(), y.stride(0), f, w.data_ptr<float>(), x.data_ptr<float>(), lp, (int)x.size(0),
-                      (int)x.size(1), (float)eps, stream()),
+                      (int)x.size(1), (float)eps, (int)groups, bp, stream()),
      "norm_resadd");
 }
 
@@ -1644,7 +1667,7 @@ void attn_prep(torch::Tensor proj, int64_t H, int64_t G, int64_t d, int64_t dv, 
 void paged_gqa_attention(torch::Tensor q, torch::Tensor kc, torch::Tensor vc, torch::Tensor bt, torch::Tensor qstart,
                          torch::Tensor qlen, torch::Tensor ctx, torch::Tensor tile_seq, torch::Tensor tile_tok0,
                          c10::optional<torch::Tensor> gate, torch::Tensor out, bool mfma, int64_t splits,
-                         c10::optional<torch::Tensor> part) {
+                         c10::optional<torch::Tensor> part, int64_t window) {
   const bool f = act_f32(q, "q");
   TORCH_CHECK(q.dim() == 3 && q.is_contiguous(), "q [T, H, d]");
   const int64_t T = q.size(0), H = q.size(1), d = q.size(2);
@@ -1652,9 +1675,10 @@ void paged_gqa_attention(torch::Tensor q, torch::Tensor kc, torch::Tensor vc, to
     TORCH_CHECK(c->is_cuda() && c->scalar_type() == q.scalar_type() && c->is_contiguous() && c->dim() == 4,
                 "paged caches K [blocks, G, block, d], V [blocks, G, dv, block] in the dtype of q");
   const int64_t G = kc.size(1), dv = vc.size(2);
-  TORCH_CHECK(G >= 1 && H % G == 0 && kc.size(3) == d && vc.size(1) == G && kc.size(0) == vc.size(0) &&
-                  kc.size(2) == vc.size(3) && dv <= 256,
-              "cache shapes; vdim <= 256");
+  const int64_t GV = vc.size(1);      // fewer value heads than key heads: neighbouring key heads share one
+  TORCH_CHECK(G >= 1 && H % G == 0 && kc.size(3) == d && GV >= 1 && G % GV == 0 && kc.size(0) == vc.size(0) &&
+                  kc.size(2) == vc.size(3) && dv <= 256 && window >= 0,
+              "cache shapes; vdim <= 256; window >= 0");
   TORCH_CHECK(!mfma || dllm_gqa_mfma_ok(f, (int)H, (int)G, (int)d, (int)dv, (int)kc.size(2)),
               "shape outside the matrix-core kernel's range");
   check_i32(bt, "block_tables");
@@ -1672,9 +1696,10 @@ void paged_gqa_attention(torch::Tensor q, torch::Tensor kc, torch::Tensor vc, to
     gp = gate->data_ptr();
     ldg = gate->stride(0);
   }
-  TORCH_CHECK(out.is_cuda() && out.scalar_type() == q.scalar_type() && out.is_contiguous() && out.dim() == 2 &&
+  const bool of32 = out.scalar_type() == torch::kFloat32;
+  TORCH_CHECK(out.is_cuda() && (of32 || out.scalar_type() == q.scalar_type()) && out.is_contiguous() && out.dim() == 2 &&
                   out.size(0) == T && out.size(1) == H * dv,
-              "out [T, H dv]");
+              "out [T, H dv] in the dtype of q or f32");
   float* pptr = nullptr;
   TORCH_CHECK(splits >= 1 && splits <= 64 && (splits == 1 || mfma), "key splits: 1..64, matrix-core kernel only");
   if (splits > 1) {
@@ -1686,9 +1711,185 @@ void paged_gqa_attention(torch::Tensor q, torch::Tensor kc, torch::Tensor vc, to
   const int rc = dllm_paged_gqa(q.data_ptr(), kc.data_ptr(), vc.data_ptr(), f, bt.data_ptr<int>(), (int)bt.stride(0),
                                 (int)kc.size(2), qstart.data_ptr<int>(), qlen.data_ptr<int>(), ctx.data_ptr<int>(),
                                 tile_seq.data_ptr<int>(), tile_tok0.data_ptr<int>(), (int)tile_seq.numel(), gp, ldg,
-                                out.data_ptr(), (int)H, (int)G, (int)d, (int)dv, (int)mfma, (int)splits, pptr, stream());
+                                out.data_ptr(), (int)H, (int)G, (int)d, (int)dv, (int)mfma, (int)splits, pptr, (int)window,
+                                (int)GV, (int)of32, stream());
   TORCH_CHECK(rc != -2, "head widths do not fit the LDS");
   ok(rc, "paged_gqa_attention");
+}
+
+// ---- differential attention, Mamba-2 / mLSTM recurrences, PolyNorm, grouped router (gqa.hip, outer_scan.hip, seqmix.hip)
+void qk_norm_prep(torch::Tensor proj, c10::optional<torch::Tensor> bias, int64_t H, int64_t G, int64_t M, int64_t d, int64_t dv,
+                  torch::Tensor qw, torch::Tensor kw, torch::Tensor cos_sin, int64_t rot, double eps, double qscale,
+                  torch::Tensor pos, torch::Tensor slots, c10::optional<torch::Tensor> kc, c10::optional<torch::Tensor> vc,
+                  torch::Tensor q) {
+  const bool f = act_f32(proj, "proj");
+  check_rows2d(proj, "proj");
+  check_f32(cos_sin, "cos_sin");
+  check_f32(qw, "q norm weight");
+  check_f32(kw, "k norm weight");
+  check_i32(pos, "positions");
+  check_i32(slots, "slots");
+  const int64_t T = proj.size(0);
+  const bool own = kc.has_value();
+  TORCH_CHECK(own == vc.has_value(), "both caches or none");
+  const int64_t cols = H * M * d + (own ? G * M * d + G * dv : 0);
+  TORCH_CHECK(H >= 1 && G >= 1 && M >= 1 && H % G == 0 && d >= 1 && dv >= 1 && proj.size(1) >= cols, "proj [T, q | k | v]");
+  TORCH_CHECK(cos_sin.dim() == 2 && rot >= 0 && rot % 2 == 0 && rot <= d && (rot == 0 || cos_sin.size(1) >= rot),
+              "rotation table");
+  TORCH_CHECK(qw.numel() == d && kw.numel() == d && pos.numel() == T && slots.numel() == T, "norm weights / positions / slots");
+  const float* bp = nullptr;
+  if (bias) {
+    check_f32(*bias, "bias");
+    TORCH_CHECK(bias->numel() == cols, "bias length");
+    bp = bias->data_ptr<float>();
+  }
+  void *kp = nullptr, *vp = nullptr;
+  int bsz = 16;
+  if (own) {
+    for (auto* c : {&*kc, &*vc})
+      TORCH_CHECK(c->is_cuda() && c->scalar_type() == proj.scalar_type() && c->is_contiguous() && c->dim() == 4,
+                  "paged caches K [blocks, G M, block, d], V [blocks, G, dv, block] in the activations' dtype");
+    TORCH_CHECK(kc->size(1) == G * M && vc->size(1) == G && kc->size(3) == d && vc->size(2) == dv &&
+                    kc->size(0) == vc->size(0) && kc->size(2) == vc->size(3),
+                "cache shapes");
+    kp = kc->data_ptr();
+    vp = vc->data_ptr();
+    bsz = (int)kc->size(2);
+  }
+  TORCH_CHECK(q.is_cuda() && q.scalar_type() == proj.scalar_type() && q.is_contiguous() && q.numel() == T * H * M * d,
+              "q [T, H M, d]");
+  ok(dllm_qk_norm_prep(proj.data_ptr(), proj.stride(0), f, bp, (int)H, (int)G, (int)M, (int)d, (int)dv, qw.data_ptr<float>(),
+                       kw.data_ptr<float>(), cos_sin.data_ptr<float>(), (int)cos_sin.size(1), (int)rot, (float)eps,
+                       (float)qscale, pos.data_ptr<int>(), slots.data_ptr<int>(), kp, vp, q.data_ptr(), (long)T, bsz, stream()),
+     "qk_norm_prep");
+}
+
+void diff_combine(torch::Tensor a, int64_t H, int64_t G, int64_t dv, double lam, double eps, double scale, torch::Tensor out) {
+  check_f32(a, "a");
+  const bool f = act_f32(out, "out");
+  TORCH_CHECK(a.dim() == 2 && a.is_contiguous() && H >= 1 && G >= 1 && H % G == 0 && a.size(1) == 2 * H * dv, "a [T, 2 H dv]");
+  TORCH_CHECK(out.is_contiguous() && out.dim() == 2 && out.size(0) == a.size(0) && out.size(1) == H * dv, "out [T, H dv]");
+  ok(dllm_diff_combine(a.data_ptr<float>(), out.data_ptr(), f, (long)a.size(0), (int)H, (int)G, (int)dv, (float)lam,
+                       (float)eps, (float)scale, stream()),
+     "diff_combine");
+}
+
+void ssd_scan(torch::Tensor xbc, torch::Tensor proj, int64_t dt_col, int64_t H, int64_t dv, int64_t N, int64_t G,
+              torch::Tensor dt_bias, torch::Tensor neg_a, torch::Tensor D, torch::Tensor state, torch::Tensor qstart,
+              torch::Tensor qlen, torch::Tensor ctx, torch::Tensor rows, torch::Tensor out) {
+  const bool f = act_f32(xbc, "xbc");
+  check_rows2d(xbc, "xbc");
+  check_rows2d(proj, "proj");
+  TORCH_CHECK(proj.scalar_type() == xbc.scalar_type() && proj.size(0) == xbc.size(0), "proj: the dtype and rows of xbc");
+  for (auto* t : {&dt_bias, &neg_a, &D}) {
+    check_f32(*t, "per-head parameter");
+    TORCH_CHECK(t->numel() == H, "per-head parameter length");
+  }
+  check_f32(state, "state");
+  check_f32(out, "out");
+  TORCH_CHECK(H >= 1 && G >= 1 && H % G == 0 && N >= 1 && dv >= 1 && xbc.size(1) >= H * dv + 2 * G * N, "xbc [T, x | B | C]");
+  TORCH_CHECK(dt_col >= 0 && proj.size(1) >= dt_col + H, "step logits outside proj");
+  TORCH_CHECK(state.is_contiguous() && state.dim() == 4 && state.size(1) == H && state.size(2) == N && state.size(3) == dv,
+              "state [slots, H, N, dv]");
+  TORCH_CHECK(out.is_contiguous() && out.dim() == 2 && out.size(0) == xbc.size(0) && out.size(1) == H * dv, "out [T, H dv] f32");
+  auto m = seq_meta(qstart, qlen, ctx, rows, state.size(0));
+  const int rc = dllm_ssd_scan(xbc.data_ptr(), xbc.stride(0), proj.data_ptr(), proj.stride(0), (int)dt_col, f, (int)H, (int)dv,
+                               (int)N, (int)G, dt_bias.data_ptr<float>(), neg_a.data_ptr<float>(), D.data_ptr<float>(),
+                               state.data_ptr<float>(), m.qstart, m.qlen, m.ctx, m.rows, m.S, out.data_ptr<float>(), stream());
+  TORCH_CHECK(rc != -2, "state size outside the kernel's range");
+  ok(rc, "ssd_scan");
+}
+
+void mlstm(torch::Tensor proj, int64_t H, int64_t d, int64_t dv, torch::Tensor gate_b, double cap, torch::Tensor state,
+           torch::Tensor nm, double eps, torch::Tensor norm_w, torch::Tensor qstart, torch::Tensor qlen, torch::Tensor ctx,
+           torch::Tensor rows, torch::Tensor raw, torch::Tensor out) {
+  const bool f = act_f32(proj, "proj");
+  check_rows2d(proj, "proj");
+  check_f32(gate_b, "gate biases");
+  check_f32(state, "state");
+  check_f32(nm, "normaliser state");
+  check_f32(norm_w, "norm weight");
+  check_f32(raw, "raw");
+  const int64_t T = proj.size(0);
+  TORCH_CHECK(H >= 1 && d >= 1 && dv >= 1 && proj.size(1) >= 2 * H * (d + dv + 1), "proj [T, q | k | v | gate | i | f]");
+  TORCH_CHECK(gate_b.numel() == 2 * H && norm_w.numel() == H * dv && cap > 0, "gate biases / norm weight / cap");
+  TORCH_CHECK(state.is_contiguous() && state.dim() == 4 && state.size(1) == H && state.size(2) == d && state.size(3) == dv,
+              "state [slots, H, d, dv]");
+  const int64_t ncb = (dv + dllm_outer_scan_cols() - 1) / dllm_outer_scan_cols();
+  TORCH_CHECK(nm.is_contiguous() && nm.dim() == 4 && nm.size(0) == state.size(0) && nm.size(1) == H && nm.size(2) == ncb &&
+                  nm.size(3) == d + 1,
+              "normaliser state [slots, H, column blocks, d + 1]");
+  TORCH_CHECK(raw.is_contiguous() && raw.numel() == T * H * dv, "raw [T, H dv] f32");
+  TORCH_CHECK(out.is_cuda() && out.scalar_type() == proj.scalar_type() && out.is_contiguous() && out.numel() == T * H * dv,
+              "out [T, H dv]");
+  auto m = seq_meta(qstart, qlen, ctx, rows, state.size(0));
+  const int rc = dllm_mlstm(proj.data_ptr(), proj.stride(0), f, (int)H, (int)d, (int)dv, gate_b.data_ptr<float>(), (float)cap,
+                            state.data_ptr<float>(), nm.data_ptr<float>(), (int)ncb, (float)eps, norm_w.data_ptr<float>(),
+                            m.qstart, m.qlen, m.ctx, m.rows, m.S, (long)T, raw.data_ptr<float>(), out.data_ptr(), stream());
+  TORCH_CHECK(rc != -2, "key width outside the kernel's range");
+  ok(rc, "mlstm");
+}
+
+void gated_group_norm(torch::Tensor y, torch::Tensor z, torch::Tensor w, int64_t groups, double eps, torch::Tensor out) {
+  check_f32(y, "y");
+  check_f32(w, "w");
+  const bool f = act_f32(z, "z");
+  check_rows2d(z, "z");
+  TORCH_CHECK(y.dim() == 2 && y.is_contiguous() && z.size(0) == y.size(0) && z.size(1) >= y.size(1) && w.numel() == y.size(1) &&
+                  groups >= 1 && y.size(1) % groups == 0,
+              "y [T, n] f32, z [T, >= n], w [n], n a multiple of groups");
+  TORCH_CHECK(out.is_cuda() && out.scalar_type() == z.scalar_type() && out.is_contiguous() && out.sizes() == y.sizes(),
+              "out [T, n] in the dtype of z");
+  ok(dllm_gated_group_norm(y.data_ptr<float>(), z.data_ptr(), z.stride(0), f, w.data_ptr<float>(), out.data_ptr(),
+                           (int)y.size(0), (int)y.size(1), (int)groups, (float)eps, stream()),
+     "gated_group_norm");
+}
+
+void polynorm(torch::Tensor z, torch::Tensor coef, double eps, torch::Tensor y) {
+  const bool f = act_f32(z, "z");
+  check_rows2d(z, "z");
+  check_f32(coef, "coef");
+  TORCH_CHECK(coef.numel() == 4, "coef = (a, b, c, e)");
+  TORCH_CHECK(y.is_cuda() && y.scalar_type() == z.scalar_type() && y.is_contiguous() && y.sizes() == z.sizes(), "y like z");
+  ok(dllm_polynorm(z.data_ptr(), z.stride(0), f, coef.data_ptr<float>(), y.data_ptr(), (long)z.size(0), (int)z.size(1),
+                   (float)eps, stream()),
+     "polynorm");
+}
+
+void group_router(torch::Tensor logits, int64_t top, int64_t count, int64_t keep, torch::Tensor ids, torch::Tensor wts) {
+  check_f32(logits, "logits");
+  check_i32(ids, "ids");
+  check_f32(wts, "wts");
+  TORCH_CHECK(logits.dim() == 2 && logits.is_contiguous(), "logits [T, E] contiguous");
+  const int64_t T = logits.size(0), E = logits.size(1);
+  TORCH_CHECK(E >= 1 && E <= 1024 && count >= 1 && E % count == 0 && keep >= 1 && keep <= count && top >= 1 &&
+                  top <= keep * (E / count),
+              "experts <= 1024, groups divide the experts, top fits the kept groups");
+  TORCH_CHECK(ids.is_contiguous() && wts.is_contiguous() && ids.numel() == T * top && wts.numel() == T * top, "ids / wts [T, top]");
+  ok(dllm_group_router(logits.data_ptr<float>(), (int)T, (int)E, (int)top, (int)count, (int)keep, ids.data_ptr<int>(),
+                       wts.data_ptr<float>(), stream()),
+     "group_router");
+}
+
+void swiglu_scale(torch::Tensor gu, torch::Tensor gate, int64_t ff, torch::Tensor y) {
+  const bool f = act_f32(gu, "gu");
+  check_f32(gate, "gate");
+  TORCH_CHECK(gu.dim() == 2 && gu.is_contiguous() && gate.dim() == 2 && gate.is_contiguous() && gate.size(0) == gu.size(0) &&
+                  ff >= 1 && gate.size(1) * 2 * ff == gu.size(1),
+              "gu [T, E 2 ff] contiguous, gate [T, E]");
+  TORCH_CHECK(y.is_cuda() && y.scalar_type() == gu.scalar_type() && y.is_contiguous() && y.dim() == 2 &&
+                  y.size(0) == gu.size(0) && y.size(1) * 2 == gu.size(1),
+              "y [T, E ff]");
+  ok(dllm_swiglu_scale(gu.data_ptr(), f, gate.data_ptr<float>(), (int)gate.size(1), (int)ff, y.data_ptr(), (long)gu.size(0),
+                       stream()),
+     "swiglu_scale");
+}
+
+void softcap(torch::Tensor x, double cap, torch::Tensor y) {
+  const bool f = act_f32(x, "x");
+  check_f32(y, "y");
+  TORCH_CHECK(x.is_contiguous() && y.is_contiguous() && x.numel() == y.numel() && cap > 0, "x / y contiguous, cap > 0");
+  ok(dllm_softcap(x.data_ptr(), f, (float)cap, y.data_ptr<float>(), (long)x.numel(), stream()), "softcap");
 }
 
 void relu2_scale(torch::Tensor x, c10::optional<torch::Tensor> gate, int64_t ff, torch::Tensor y) {
@@ -1789,8 +1990,19 @@ void latent_attention(torch::Tensor qa, torch::Tensor q, int64_t dim, int64_t ro
 }  // namespace
 
 PYBIND11_MODULE(_hip_kernels, m) {
-  m.def("rms_rows", &rms_rows);
-  m.def("norm_resadd", &norm_resadd);
+  m.def("rms_rows", &rms_rows, py::arg("x"), py::arg("w"), py::arg("y"), py::arg("eps"), py::arg("groups") = 1);
+  m.def("norm_resadd", &norm_resadd, py::arg("y"), py::arg("w"), py::arg("eps"), py::arg("x"), py::arg("x_lp"),
+        py::arg("groups") = 1, py::arg("bias") = py::none());
+  m.def("polynorm", &polynorm);
+  m.def("group_router", &group_router);
+  m.def("swiglu_scale", &swiglu_scale);
+  m.def("softcap", &softcap);
+  m.def("gated_group_norm", &gated_group_norm);
+  m.def("outer_scan_cols", []() { return dllm_outer_scan_cols(); });
+  m.def("ssd_scan", &ssd_scan);
+  m.def("mlstm", &mlstm);
+  m.def("qk_norm_prep", &qk_norm_prep);
+  m.def("diff_combine", &diff_combine);
   m.def("causal_conv_silu", &causal_conv_silu, py::arg("x"), py::arg("w"), py::arg("b"), py::arg("state"), py::arg("qstart"),
         py::arg("qlen"), py::arg("ctx"), py::arg("rows"), py::arg("y"), py::arg("refill") = false);
   m.def("selective_scan", &selective_scan);
@@ -1811,7 +2023,7 @@ PYBIND11_MODULE(_hip_kernels, m) {
   m.def("paged_gqa_attention", &paged_gqa_attention, py::arg("q"), py::arg("k_cache"), py::arg("v_cache"),
         py::arg("block_tables"), py::arg("qstart"), py::arg("qlen"), py::arg("ctx"), py::arg("tile_seq"),
         py::arg("tile_tok0"), py::arg("gate"), py::arg("out"), py::arg("mfma"), py::arg("splits") = 1,
-        py::arg("part") = py::none());
+        py::arg("part") = py::none(), py::arg("window") = 0);
   m.def("gqa_tile_tokens",
         [](int64_t H, int64_t G, bool mfma) { return (int64_t)dllm_gqa_tile_tokens((int)H, (int)G, (int)mfma); });
   m.def("gqa_mfma_ok", [](bool f32, int64_t H, int64_t G, int64_t d, int64_t dv, int64_t bs) {

@@ -3,6 +3,10 @@
 //   attn_prep   one workgroup per token: rotate-half positions on the first `rot` dims of every q / k
 //               head, each head to unit RMS (f32), q times a per-head scale; k and v go to their
 //               page slots, q to a dense [T, H, d] buffer.
+//   qk_norm_prep  attention inputs with biases, a weighted RMS norm of every q / k vector before its
+//               rotation, and `maps` score maps per head (differential attention: 2): query rows of
+//               one key/value head leave ordered (map, head in group), so the grouped-query kernels
+//               below pair them with key head (kv head, map); diff_combine merges the two maps.
 //   paged_gqa   one workgroup per (tile of new tokens, key/value head, group of <= 16 query heads):
 //               its rows are tokens x query heads of the group (<= 16).  Keys are walked in tiles
 //               staged in LDS as f32; a lane owns a key for the scores (one K read feeds the wave's
@@ -81,6 +85,86 @@ __global__ void __launch_bounds__(256) attn_prep_kernel(const T* __restrict__ pr
   }
 }
 
+// One wave per q / k vector (head, map): bias, weighted RMS norm over d, rotate-half positions on the
+// first `rot` dims, q times `qscale`.  Query unit (h, m) of key/value head g = h / R leaves as row
+// g M R + m R + h % R of q [T, H M, d]; key unit (g, m) goes to key head g M + m of the page.
+template <typename T>
+__global__ void __launch_bounds__(256) qk_norm_prep_kernel(const T* __restrict__ proj, long ld, const float* __restrict__ bias,
+                                                           int H, int G, int M, int d, int dv,
+                                                           const float* __restrict__ qw, const float* __restrict__ kw,
+                                                           const float* __restrict__ cos_sin, int tab_w, int rot, float eps,
+                                                           float qscale, const int* __restrict__ pos,
+                                                           const int* __restrict__ slots, T* __restrict__ kc,
+                                                           T* __restrict__ vc, T* __restrict__ q, int BSZ) {
+  const long tok = blockIdx.x;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const T* r = proj + tok * ld;
+  const int slot = kc ? slots[tok] : -1;
+  const long blk = slot >= 0 ? slot / BSZ : 0;
+  const int off = slot >= 0 ? slot % BSZ : 0;
+  const int half = rot >> 1;
+  const float* cs = cos_sin + (long)pos[tok] * tab_w;
+  const int nq = H * M, nk = kc ? G * M : 0;
+  const int u = blockIdx.y * 4 + wave;     // q units, then k units, are consecutive in the projection
+  if (u < nq + nk && (u < nq || slot >= 0)) {
+    const bool is_q = u < nq;
+    const T* x = r + (long)u * d;
+    const float* b = bias ? bias + (long)u * d : nullptr;
+    const float* w = is_q ? qw : kw;
+    float ss = 0.f;
+    for (int i = lane; i < d; i += 64) {
+      const float v = ldf(x + i) + (b ? b[i] : 0.f);
+      ss += v * v;
+    }
+    const float sc = 1.f / sqrtf(wave_sum(ss) / (float)d + eps);
+    T* dst;
+    if (is_q) {
+      const int h = u / M, m = u % M, R = H / G;
+      dst = q + (tok * nq + (long)(h / R) * M * R + m * R + h % R) * d;
+    } else {
+      dst = kc + ((blk * nk + (u - nq)) * BSZ + off) * d;
+    }
+    const float os = is_q ? qscale : 1.f;
+    for (int i = lane; i < d; i += 64) {
+      float v = (ldf(x + i) + (b ? b[i] : 0.f)) * sc * w[i];
+      if (i < rot) {
+        const int f = i < half ? i : i - half;
+        const int j = i < half ? i + half : i - half;
+        const float c = cs[f], sn = cs[half + f];
+        const float p = (ldf(x + j) + (b ? b[j] : 0.f)) * sc * w[j];
+        v = i < half ? v * c - p * sn : v * c + p * sn;
+      }
+      stf(dst + i, v * os);
+    }
+  }
+  if (slot >= 0) {   // values: this workgroup's share of the G * dv entries
+    const long vo = (long)(nq + nk) * d;
+    for (int i = blockIdx.y * 256 + threadIdx.x; i < G * dv; i += gridDim.y * 256)
+      stf(vc + ((blk * G + i / dv) * dv + i % dv) * BSZ + off, ldf(r + vo + i) + (bias ? bias[vo + i] : 0.f));
+  }
+}
+
+// a [T, G, 2, R, dv] f32 (the two maps' outputs) -> out [T, G R, dv] = unit-RMS(a1 - lam a2) * scale:
+// one wave per (token, head)
+template <typename T>
+__global__ void __launch_bounds__(256) diff_combine_kernel(const float* __restrict__ a, T* __restrict__ out, long units, int H,
+                                                           int G, int dv, float lam, float eps, float scale) {
+  const long u = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63;
+  if (u >= units) return;
+  const long tok = u / H;
+  const int h = (int)(u % H), R = H / G;
+  const float* a1 = a + ((tok * G + h / R) * 2 * R + h % R) * dv;
+  const float* a2 = a1 + (long)R * dv;
+  float ss = 0.f;
+  for (int i = lane; i < dv; i += 64) {
+    const float o = a1[i] - lam * a2[i];
+    ss += o * o;
+  }
+  const float sc = scale / sqrtf(wave_sum(ss) / (float)dv + eps);
+  for (int i = lane; i < dv; i += 64) stf(out + u * dv + i, (a1[i] - lam * a2[i]) * sc);
+}
+
 constexpr int GA_ROWS = 16;   // rows per workgroup: 4 per wave
 
 // KT keys per tile (64, or 32 when the tile would not fit the LDS), NJ = ceil(dv / 64)
@@ -91,7 +175,10 @@ __global__ void __launch_bounds__(256) paged_gqa_kernel(const T* __restrict__ q,
                                                         const int* __restrict__ qlen, const int* __restrict__ ctx,
                                                         const int* __restrict__ tile_seq, const int* __restrict__ tile_tok0,
                                                         const T* __restrict__ gate, long ldg, T* __restrict__ out, int H,
-                                                        int G, int d, int dv, int TQ, int KT) {
+                                                        int G, int d, int dv, int TQ, int KT, int win, int GV,
+                                                        float* __restrict__ out32) {
+  // win > 0: a row at position p sees keys p - win < j <= p.  GV value heads: key head g reads value
+  // head g / (G / GV).  out32: the output stays f32.
   extern __shared__ float sm[];
   const int s = tile_seq[blockIdx.x];
   const int n = qlen[s];
@@ -127,7 +214,9 @@ __global__ void __launch_bounds__(256) paged_gqa_kernel(const T* __restrict__ q,
   }
   const int last = p0 + tok0 + nq - 1;   // the newest key any row sees
   const int* btr = bt + (long)s * bt_ld;
-  for (int k0 = 0; k0 <= last; k0 += KT) {
+  const int gv = g / (G / GV);
+  const int first = win > 0 ? max(0, p0 + tok0 - win + 1) : 0;   // the oldest key any row sees
+  for (int k0 = first / KT * KT; k0 <= last; k0 += KT) {
     const int nk = min(KT, last + 1 - k0);
     __syncthreads();   // the previous tile is consumed (and Qs is written)
     for (int e = tid; e < KT * d; e += 256) {
@@ -144,7 +233,7 @@ __global__ void __launch_bounds__(256) paged_gqa_kernel(const T* __restrict__ q,
       float v = 0.f;
       if (kk < nk) {
         const int pk = k0 + kk;
-        v = ldf(vc + (((long)btr[pk / BSZ] * G + g) * dv + jx) * BSZ + pk % BSZ);
+        v = ldf(vc + (((long)btr[pk / BSZ] * GV + gv) * dv + jx) * BSZ + pk % BSZ);
       }
       Vs[e] = v;
     }
@@ -163,7 +252,7 @@ __global__ void __launch_bounds__(256) paged_gqa_kernel(const T* __restrict__ q,
     const int pk = k0 + lane;
 #pragma unroll
     for (int x = 0; x < 4; ++x) {
-      const bool vis = lane < nk && pk <= rpos[x];
+      const bool vis = lane < nk && pk <= rpos[x] && (win <= 0 || pk > rpos[x] - win);
       const float sv = vis ? sc[x] : -INFINITY;
       const float mn = fmaxf(m[x], wave_max(sv));
       float p = 0.f, f = 1.f;
@@ -204,7 +293,8 @@ __global__ void __launch_bounds__(256) paged_gqa_kernel(const T* __restrict__ q,
       if (jx >= dv) continue;
       float o = O[x][jj] * inv;
       if (gate) o *= 1.f / (1.f + expf(-ldf(gate + tok * ldg + (long)h * dv + jx)));
-      stf(out + tok * ((long)H * dv) + (long)h * dv + jx, o);
+      if (out32) out32[tok * ((long)H * dv) + (long)h * dv + jx] = o;
+      else stf(out + tok * ((long)H * dv) + (long)h * dv + jx, o);
     }
   }
 }
@@ -242,7 +332,8 @@ __global__ void __launch_bounds__(256) paged_gqa_mfma_kernel(const u16* __restri
                                                              const int* __restrict__ tile_seq,
                                                              const int* __restrict__ tile_tok0, const u16* __restrict__ gate,
                                                              long ldg, u16* __restrict__ out, int H, int G, int d, int dv,
-                                                             int TQ, int splits, float* __restrict__ part) {
+                                                             int TQ, int splits, float* __restrict__ part, int win, int GV,
+                                                             float* __restrict__ out32) {
   constexpr int DS = SZ / 32, VB = SZ / 16, NKB = GM_KT / 16;
   constexpr int KSTR = SZ + 8, VSTR = GM_KT + 8, PSTR = GM_KT + 8;
   extern __shared__ __attribute__((aligned(16))) unsigned char smraw[];
@@ -289,6 +380,8 @@ __global__ void __launch_bounds__(256) paged_gqa_mfma_kernel(const u16* __restri
   const int wave_last = 16 * wave < nrows ? p0 + tok0 + (min(16 * wave + 15, nrows - 1)) / R : -1;
   // the oldest row of the wave; idle rows (past nrows) are masked, so a wave that has any never skips the mask
   const int wave_first = 16 * wave + 15 < nrows ? p0 + tok0 + (16 * wave) / R : -1;
+  // with a window: the wave's oldest live row (tiles wholly before its window are skipped)
+  const int wave_old = 16 * wave < nrows ? p0 + tok0 + (16 * wave) / R : 0x3fffffff;
   const int last = p0 + tok0 + nq - 1;   // the newest key any row sees
   const int* btr = bt + (long)s * bt_ld;
   constexpr int KCH = SZ / 8;            // 16-byte chunks of a staged key row
@@ -301,7 +394,8 @@ __global__ void __launch_bounds__(256) paged_gqa_mfma_kernel(const u16* __restri
   long koff[NF], voff[NF];
   int kkey[NF], vpg[NF];
   bool kon[NF], von[NF];
-  const long kpage = (long)G * GM_BS * d, vpage = (long)G * dv * GM_BS;
+  const long kpage = (long)G * GM_BS * d, vpage = (long)GV * dv * GM_BS;
+  const int gv = g / (G / GV);
 #pragma unroll
   for (int f = 0; f < NF; ++f) {
     const int e = tid + 256 * f;
@@ -312,7 +406,7 @@ __global__ void __launch_bounds__(256) paged_gqa_mfma_kernel(const u16* __restri
     const int j = e / (GM_KT / 8), cc = e % (GM_KT / 8);
     vpg[f] = cc >> 1;
     von[f] = j < dv;
-    voff[f] = ((long)g * dv + j) * GM_BS + 8 * (cc & 1);
+    voff[f] = ((long)gv * dv + j) * GM_BS + 8 * (cc & 1);
   }
   auto fetch = [&](int k0) {
     const int nk = min(GM_KT, last + 1 - k0);
@@ -327,9 +421,10 @@ __global__ void __launch_bounds__(256) paged_gqa_mfma_kernel(const u16* __restri
   };
   // small grids (decode steps) split a row's key tiles over `splits` workgroups; each leaves its
   // running maximum, sum and unnormalised output in `part`, gqa_combine merges them
-  const int ntiles = last / GM_KT + 1;
-  const int kbeg = (int)((long)ntiles * blockIdx.z / splits) * GM_KT;
-  const int kend = (int)((long)ntiles * (blockIdx.z + 1) / splits) * GM_KT;   // exclusive
+  const int tfirst = win > 0 ? max(0, p0 + tok0 - win + 1) / GM_KT : 0;   // the oldest tile any row sees
+  const int ntiles = last / GM_KT + 1 - tfirst;
+  const int kbeg = (tfirst + (int)((long)ntiles * blockIdx.z / splits)) * GM_KT;
+  const int kend = (tfirst + (int)((long)ntiles * (blockIdx.z + 1) / splits)) * GM_KT;   // exclusive
   if (kbeg < kend) fetch(kbeg);
   for (int k0 = kbeg; k0 < kend; k0 += GM_KT) {
     __syncthreads();   // the previous tile is consumed
@@ -344,6 +439,7 @@ __global__ void __launch_bounds__(256) paged_gqa_mfma_kernel(const u16* __restri
     if (k0 + GM_KT < kend) fetch(k0 + GM_KT);   // the next tile's loads fly under this tile's products
     __syncthreads();
     if (k0 > wave_last) continue;   // this wave's rows see nothing of the tile (the barriers above are uniform)
+    if (win > 0 && k0 + GM_KT - 1 <= wave_old - win) continue;   // ... or the tile lies before every row's window
     f32x4 sacc[NKB];
 #pragma unroll
     for (int kb = 0; kb < NKB; ++kb) {
@@ -360,12 +456,13 @@ __global__ void __launch_bounds__(256) paged_gqa_mfma_kernel(const u16* __restri
     float alpha[4];
     const int key0 = k0 + 4 * lr;
     // a tile below the wave's oldest row needs no mask (wave-uniform)
-    const bool full = k0 + GM_KT - 1 <= wave_first;
+    const bool full = k0 + GM_KT - 1 <= wave_first && (win <= 0 || k0 > wave_last - win);
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       float sv[NKB];
 #pragma unroll
-      for (int kb = 0; kb < NKB; ++kb) sv[kb] = (full || key0 + kb <= rpos[i]) ? sacc[kb][i] : -INFINITY;
+      for (int kb = 0; kb < NKB; ++kb)
+        sv[kb] = (full || (key0 + kb <= rpos[i] && (win <= 0 || key0 + kb > rpos[i] - win))) ? sacc[kb][i] : -INFINITY;
       float mx = fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3]));
       mx = row16_max(mx);
       const float mn = fmaxf(m[i], mx);
@@ -433,7 +530,8 @@ __global__ void __launch_bounds__(256) paged_gqa_mfma_kernel(const u16* __restri
       if (jx >= dv) continue;
       float o = acc[cb][i] * inv;
       if (gate) o *= 1.f / (1.f + expf(-bf2f(gate[tok * ldg + (long)h * dv + jx])));
-      out[tok * ((long)H * dv) + (long)h * dv + jx] = f2bf(o);
+      if (out32) out32[tok * ((long)H * dv) + (long)h * dv + jx] = o;
+      else out[tok * ((long)H * dv) + (long)h * dv + jx] = f2bf(o);
     }
   }
 }
@@ -443,7 +541,8 @@ __global__ void __launch_bounds__(256) gqa_combine_kernel(const float* __restric
                                                           const int* __restrict__ qstart, const int* __restrict__ qlen,
                                                           const int* __restrict__ tile_seq,
                                                           const int* __restrict__ tile_tok0, const u16* __restrict__ gate,
-                                                          long ldg, u16* __restrict__ out, int H, int G, int dv, int TQ) {
+                                                          long ldg, u16* __restrict__ out, int H, int G, int dv, int TQ,
+                                                          float* __restrict__ out32) {
   const int s = tile_seq[blockIdx.x];
   const int n = qlen[s], tok0 = tile_tok0[blockIdx.x];
   if (n <= 0 || tok0 >= n) return;
@@ -473,7 +572,8 @@ __global__ void __launch_bounds__(256) gqa_combine_kernel(const float* __restric
       if (!on) continue;
       o /= L;
       if (gate) o *= 1.f / (1.f + expf(-bf2f(gate[tok * ldg + (long)h * dv + jx])));
-      out[tok * ((long)H * dv) + (long)h * dv + jx] = f2bf(o);
+      if (out32) out32[tok * ((long)H * dv) + (long)h * dv + jx] = o;
+      else out[tok * ((long)H * dv) + (long)h * dv + jx] = f2bf(o);
     }
   }
 }
@@ -494,18 +594,19 @@ long gqa_lds(int d, int dv, int KT) { return 4L * (GA_ROWS * d + (long)KT * (d |
 template <typename T, int NJ>
 int launch_gqa(dim3 grid, long lds, hipStream_t st, const T* q, const T* kc, const T* vc, const int* bt, int bt_ld, int BSZ,
                const int* qstart, const int* qlen, const int* ctx, const int* tile_seq, const int* tile_tok0, const T* gate,
-               long ldg, T* out, int H, int G, int d, int dv, int TQ, int KT) {
+               long ldg, T* out, int H, int G, int d, int dv, int TQ, int KT, int win, int GV, float* out32) {
   ENSURE_LDS((paged_gqa_kernel<T, NJ>), lds);
   hipLaunchKernelGGL((paged_gqa_kernel<T, NJ>), grid, dim3(256), lds, st, q, kc, vc, bt, bt_ld, BSZ, qstart, qlen, ctx, tile_seq,
-                     tile_tok0, gate, ldg, out, H, G, d, dv, TQ, KT);
+                     tile_tok0, gate, ldg, out, H, G, d, dv, TQ, KT, win, GV, out32);
   return (int)hipGetLastError();
 }
 
 template <typename T>
 int launch_gqa_t(int nj, dim3 grid, long lds, hipStream_t st, const void* q, const void* kc, const void* vc, const int* bt,
                  int bt_ld, int BSZ, const int* qstart, const int* qlen, const int* ctx, const int* tile_seq,
-                 const int* tile_tok0, const void* gate, long ldg, void* out, int H, int G, int d, int dv, int TQ, int KT) {
-#define GQA(NJ) return launch_gqa<T, NJ>(grid, lds, st, (const T*)q, (const T*)kc, (const T*)vc, bt, bt_ld, BSZ, qstart, qlen, ctx, tile_seq, tile_tok0, (const T*)gate, ldg, (T*)out, H, G, d, dv, TQ, KT)
+                 const int* tile_tok0, const void* gate, long ldg, void* out, int H, int G, int d, int dv, int TQ, int KT,
+                 int win, int GV, float* out32) {
+#define GQA(NJ) return launch_gqa<T, NJ>(grid, lds, st, (const T*)q, (const T*)kc, (const T*)vc, bt, bt_ld, BSZ, qstart, qlen, ctx, tile_seq, tile_tok0, (const T*)gate, ldg, (T*)out, H, G, d, dv, TQ, KT, win, GV, out32)
   if (nj <= 1) GQA(1);
   if (nj <= 2) GQA(2);
   GQA(4);
@@ -544,9 +645,10 @@ extern "C" int dllm_gqa_tile_tokens(int H, int G, int mfma) {
 extern "C" int dllm_paged_gqa(const void* q, const void* kc, const void* vc, int f32, const int* bt, int bt_ld, int BSZ,
                               const int* qstart, const int* qlen, const int* ctx, const int* tile_seq, const int* tile_tok0,
                               int n_tiles, const void* gate, long ldg, void* out, int H, int G, int d, int dv, int mfma,
-                              int splits, float* part, hipStream_t st) {
+                              int splits, float* part, int win, int GV, int out_f32, hipStream_t st) {
   if (n_tiles <= 0) return 0;
-  if (G < 1 || H % G || dv > 256 || d < 1) return -1;
+  if (G < 1 || H % G || dv > 256 || d < 1 || GV < 1 || G % GV || win < 0) return -1;
+  float* out32 = out_f32 ? (float*)out : nullptr;
   if (mfma) {
     if (!dllm_gqa_mfma_ok(f32, H, G, d, dv, BSZ)) return -1;
     const int sz = d > dv ? d : dv;
@@ -560,14 +662,14 @@ extern "C" int dllm_paged_gqa(const void* q, const void* kc, const void* vc, int
     ENSURE_LDS(paged_gqa_mfma_kernel<SZ>, lds);                                                                          \
     hipLaunchKernelGGL(paged_gqa_mfma_kernel<SZ>, grid, dim3(256), lds, st, (const u16*)q, (const u16*)kc, (const u16*)vc, bt, \
                        bt_ld, qstart, qlen, ctx, tile_seq, tile_tok0, (const u16*)gate, ldg, (u16*)out, H, G, d, dv, TQ, \
-                       splits, pp);                                                                                      \
+                       splits, pp, win, GV, out32);                                                                      \
   } while (0)
     if (sz <= 64) GQM(64); else if (sz <= 128) GQM(128); else GQM(256);
 #undef GQM
     if (pp) {
       const int rows = (TQ * (H / G) < GM_ROWS ? TQ * (H / G) : GM_ROWS);
       hipLaunchKernelGGL(gqa_combine_kernel, dim3(n_tiles, G, (rows + 3) / 4), dim3(256), 0, st, pp, splits, qstart, qlen,
-                         tile_seq, tile_tok0, (const u16*)gate, ldg, (u16*)out, H, G, dv, TQ);
+                         tile_seq, tile_tok0, (const u16*)gate, ldg, (u16*)out, H, G, dv, TQ, out32);
     }
     return (int)hipGetLastError();
   }
@@ -581,7 +683,37 @@ extern "C" int dllm_paged_gqa(const void* q, const void* kc, const void* vc, int
   const int TQ = dllm_gqa_tile_tokens(H, G, 0);
   if (f32)
     return launch_gqa_t<float>(nj, grid, lds, st, q, kc, vc, bt, bt_ld, BSZ, qstart, qlen, ctx, tile_seq, tile_tok0, gate, ldg,
-                               out, H, G, d, dv, TQ, KT);
+                               out, H, G, d, dv, TQ, KT, win, GV, out32);
   return launch_gqa_t<u16>(nj, grid, lds, st, q, kc, vc, bt, bt_ld, BSZ, qstart, qlen, ctx, tile_seq, tile_tok0, gate, ldg, out,
-                           H, G, d, dv, TQ, KT);
+                           H, G, d, dv, TQ, KT, win, GV, out32);
+}
+
+extern "C" int dllm_qk_norm_prep(const void* proj, long ld, int f32, const float* bias, int H, int G, int M, int d, int dv,
+                                 const float* qw, const float* kw, const float* cos_sin, int tab_w, int rot, float eps,
+                                 float qscale, const int* pos, const int* slots, void* kc, void* vc, void* q, long T, int BSZ,
+                                 hipStream_t st) {
+  if (T <= 0) return 0;
+  if (rot < 0 || rot > d || (rot & 1) || rot > tab_w || H < 1 || G < 1 || H % G || M < 1) return -1;
+  const int units = H * M + (kc ? G * M : 0);
+  const dim3 grid((unsigned)T, (units + 3) / 4);
+  if (f32)
+    hipLaunchKernelGGL(qk_norm_prep_kernel<float>, grid, dim3(256), 0, st, (const float*)proj, ld, bias, H, G, M, d, dv, qw, kw,
+                       cos_sin, tab_w, rot, eps, qscale, pos, slots, (float*)kc, (float*)vc, (float*)q, BSZ);
+  else
+    hipLaunchKernelGGL(qk_norm_prep_kernel<u16>, grid, dim3(256), 0, st, (const u16*)proj, ld, bias, H, G, M, d, dv, qw, kw,
+                       cos_sin, tab_w, rot, eps, qscale, pos, slots, (u16*)kc, (u16*)vc, (u16*)q, BSZ);
+  return (int)hipGetLastError();
+}
+
+extern "C" int dllm_diff_combine(const float* a, void* out, int f32, long T, int H, int G, int dv, float lam, float eps,
+                                 float scale, hipStream_t st) {
+  if (T <= 0) return 0;
+  if (H < 1 || G < 1 || H % G) return -1;
+  const long units = T * H;
+  const dim3 grid((unsigned)((units + 3) / 4));
+  if (f32)
+    hipLaunchKernelGGL(diff_combine_kernel<float>, grid, dim3(256), 0, st, a, (float*)out, units, H, G, dv, lam, eps, scale);
+  else
+    hipLaunchKernelGGL(diff_combine_kernel<u16>, grid, dim3(256), 0, st, a, (u16*)out, units, H, G, dv, lam, eps, scale);
+  return (int)hipGetLastError();
 }

@@ -18,6 +18,10 @@
 //                    layer results, plus the normed input of the next layer; gelu_erf; conv_refill
 //   relu2_scale      relu(x)^2 (* a per-(token, expert) gate): squared-ReLU experts, dense form
 //   dense_gate       top-k (id, weight) pairs -> [T, E] gate matrix
+//   polynorm         a N(z) + b N(z^2) + c N(z^3) + e per row (N: to unit RMS), one workgroup per row
+//   group_router     sigmoid scores, group-limited top-k, weights = scores: one wave per token
+//   swiglu_scale     silu(gate) * up * a per-(token, expert) weight: SwiGLU experts, dense form
+//   softcap          cap * tanh(x / cap) in f32;  gated_group_norm: rmsnorm in parts of y silu(z)
 //
 // Activations are bf16 or f32 (template T = u16 / float); every sum, state, norm and gate is f32.
 // Sequence metadata: qstart / qlen / ctx / rows per sequence (int32); a sequence with qlen 0 is
@@ -659,6 +663,139 @@ __global__ void __launch_bounds__(256) dense_gate_kernel(const int* __restrict__
   if (e >= 0 && e < E) g[(p / k) * E + e] = wts[p];   // a token's k experts are distinct
 }
 
+
+// ---------------------------------------------------------------- PolyNorm, grouped sigmoid router, SwiGLU dense form, softcap
+// y = a N(z) + b N(z^2) + c N(z^3) + e per row, N(u) = u / sqrt(mean(u^2) + eps): one workgroup per row
+template <typename T>
+__global__ void __launch_bounds__(256) polynorm_kernel(const T* __restrict__ z, long ldz, const float* __restrict__ coef,
+                                                       T* __restrict__ y, int n, float eps) {
+  __shared__ float red[16];
+  const long row = blockIdx.x;
+  const T* zr = z + row * ldz;
+  float s1 = 0.f, s2 = 0.f, s3 = 0.f;
+  for (int i = threadIdx.x; i < n; i += 256) {
+    const float v = ldf(zr + i), v2 = v * v;
+    s1 += v2;
+    s2 += v2 * v2;
+    s3 += v2 * v2 * v2;
+  }
+  const float inv = 1.f / (float)n;
+  const float r1 = coef[0] / sqrtf(block_sum(s1, red) * inv + eps);
+  const float r2 = coef[1] / sqrtf(block_sum(s2, red) * inv + eps);
+  const float r3 = coef[2] / sqrtf(block_sum(s3, red) * inv + eps);
+  const float e = coef[3];
+  for (int i = threadIdx.x; i < n; i += 256) {
+    const float v = ldf(zr + i);
+    stf(y + row * (long)n + i, v * (r1 + v * (r2 + v * r3)) + e);
+  }
+}
+
+// (value, index) maximum over the wave; equal values: the lower index
+__device__ __forceinline__ void wave_argmax(float& v, int& idx) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    const float ov = __shfl_xor(v, o, 64);
+    const int oi = __shfl_xor(idx, o, 64);
+    if (ov > v || (ov == v && oi < idx)) { v = ov; idx = oi; }
+  }
+}
+
+constexpr int ROUTER_MAX_E = 1024;
+
+// one wave per token: sigmoid scores, a group's score = the sum of its two best, the `top` best
+// experts inside the `keep` best groups; weights are the scores themselves
+__global__ void __launch_bounds__(256) group_router_kernel(const float* __restrict__ logits, int T, int E, int top, int count,
+                                                           int keep, int* __restrict__ ids, float* __restrict__ wts) {
+  __shared__ float sc_[4][ROUTER_MAX_E];
+  __shared__ float gs_[4][ROUTER_MAX_E];
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int t = blockIdx.x * 4 + wave;
+  if (t >= T) return;
+  float* sc = sc_[wave];
+  float* gs = gs_[wave];     // group score; -2: group chosen, experts allowed
+  for (int e = lane; e < E; e += 64) sc[e] = 1.f / (1.f + expf(-logits[(long)t * E + e]));
+  const int per = E / count;
+  const bool limited = count > 1 && keep < count;
+  if (limited) {
+    __builtin_amdgcn_wave_barrier();
+    for (int g = lane; g < count; g += 64) {
+      float a = -1.f, b = -1.f;     // the two best (scores are in (0, 1))
+      for (int j = 0; j < per; ++j) {
+        const float v = sc[g * per + j];
+        if (v > a) { b = a; a = v; } else if (v > b) b = v;
+      }
+      gs[g] = a + (per > 1 ? b : 0.f);
+    }
+    __builtin_amdgcn_wave_barrier();
+    for (int kk = 0; kk < keep; ++kk) {
+      float bv = -1.f;
+      int bi = 0x7fffffff;
+      for (int g = lane; g < count; g += 64) {
+        const float v = gs[g];
+        if (v > bv) { bv = v; bi = g; }
+      }
+      wave_argmax(bv, bi);
+      if (lane == 0) gs[bi] = -2.f;
+      __builtin_amdgcn_wave_barrier();
+    }
+  }
+  for (int j = 0; j < top; ++j) {
+    float bv = -1.f;
+    int bi = 0x7fffffff;
+    for (int e = lane; e < E; e += 64) {
+      const float v = sc[e];
+      if (v > bv && (!limited || gs[e / per] == -2.f)) { bv = v; bi = e; }
+    }
+    wave_argmax(bv, bi);
+    if (lane == 0) {
+      ids[(long)t * top + j] = bi;
+      wts[(long)t * top + j] = bv;
+      sc[bi] = -1.f;     // taken
+    }
+    __builtin_amdgcn_wave_barrier();
+  }
+}
+
+// gu [rows, E 2 ff] (per expert: gate columns, then up columns) -> y [rows, E ff] = silu(gate) up gate[row, expert]
+template <typename T>
+__global__ void __launch_bounds__(256) swiglu_scale_kernel(const T* __restrict__ gu, const float* __restrict__ gate, int E,
+                                                           int ff, T* __restrict__ y, long total) {
+  const long i = (long)blockIdx.x * 256 + threadIdx.x;
+  if (i >= total) return;
+  const long n = (long)E * ff, row = i / n;
+  const int c = (int)(i % n), e = c / ff, j = c % ff;
+  const float w = gate[row * E + e];
+  float v = 0.f;
+  if (w != 0.f) {
+    const T* p = gu + row * 2 * n + (long)e * 2 * ff + j;
+    v = silu_f(ldf(p)) * ldf(p + ff) * w;
+  }
+  stf(y + i, v);
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256) softcap_kernel(const T* __restrict__ x, float cap, float* __restrict__ y, long n) {
+  const long i = (long)blockIdx.x * 256 + threadIdx.x;
+  if (i < n) y[i] = cap * tanhf(ldf(x + i) / cap);
+}
+
+// out = rmsnorm over each of `groups` parts of (y silu(z)), times w: a wave per (row, part)
+template <typename T>
+__global__ void __launch_bounds__(256) gated_group_norm_kernel(const float* __restrict__ y, const T* __restrict__ z, long ldz,
+                                                               const float* __restrict__ w, T* __restrict__ out, int rows,
+                                                               int n, int groups, float eps) {
+  const int unit = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+  if (unit >= rows * groups) return;
+  const int row = unit / groups, c0 = (unit % groups) * n;
+  const float* yr = y + (long)row * n * groups + c0;
+  const T* zr = z + (long)row * ldz + c0;
+  float s = 0.f;
+  for (int i = lane; i < n; i += 64) { const float v = yr[i] * silu_f(ldf(zr + i)); s += v * v; }
+  const float r = 1.f / sqrtf(wave_sum(s) / (float)n + eps);
+  T* o = out + (long)row * n * groups + c0;
+  for (int i = lane; i < n; i += 64) stf(o + i, yr[i] * silu_f(ldf(zr + i)) * r * w[c0 + i]);
+}
+
 }  // namespace
 
 // Raise a kernel's dynamic-LDS limit when a launch needs more than it has been given so far (once per
@@ -890,5 +1027,56 @@ extern "C" int dllm_dense_gate(const int* ids, const float* wts, float* g, long 
   const long P = T * k;
   if (P <= 0) return 0;
   hipLaunchKernelGGL(dense_gate_kernel, dim3((int)((P + 255) / 256)), dim3(256), 0, st, ids, wts, g, P, k, E);
+  return (int)hipGetLastError();
+}
+
+extern "C" int dllm_polynorm(const void* z, long ldz, int f32, const float* coef, void* y, long rows, int n, float eps,
+                             hipStream_t st) {
+  if (rows <= 0 || n <= 0) return rows == 0 ? 0 : -1;
+  BY_T(f32,
+       hipLaunchKernelGGL(polynorm_kernel<u16>, dim3((unsigned)rows), dim3(256), 0, st, (const u16*)z, ldz, coef, (u16*)y, n, eps),
+       hipLaunchKernelGGL(polynorm_kernel<float>, dim3((unsigned)rows), dim3(256), 0, st, (const float*)z, ldz, coef, (float*)y, n, eps))
+  return (int)hipGetLastError();
+}
+
+extern "C" int dllm_group_router(const float* logits, int T, int E, int top, int count, int keep, int* ids, float* wts,
+                                 hipStream_t st) {
+  if (T <= 0) return 0;
+  if (E < 1 || E > ROUTER_MAX_E || count < 1 || E % count || keep < 1 || keep > count || top < 1 ||
+      top > keep * (E / count))
+    return -1;
+  hipLaunchKernelGGL(group_router_kernel, dim3((T + 3) / 4), dim3(256), 0, st, logits, T, E, top, count, keep, ids, wts);
+  return (int)hipGetLastError();
+}
+
+extern "C" int dllm_swiglu_scale(const void* gu, int f32, const float* gate, int E, int ff, void* y, long rows,
+                                 hipStream_t st) {
+  const long total = rows * E * ff;
+  if (total <= 0) return 0;
+  const dim3 g((unsigned)((total + 255) / 256));
+  BY_T(f32,
+       hipLaunchKernelGGL(swiglu_scale_kernel<u16>, g, dim3(256), 0, st, (const u16*)gu, gate, E, ff, (u16*)y, total),
+       hipLaunchKernelGGL(swiglu_scale_kernel<float>, g, dim3(256), 0, st, (const float*)gu, gate, E, ff, (float*)y, total))
+  return (int)hipGetLastError();
+}
+
+extern "C" int dllm_softcap(const void* x, int f32, float cap, float* y, long n, hipStream_t st) {
+  if (n <= 0) return 0;
+  if (!(cap > 0.f)) return -1;
+  const dim3 g((unsigned)((n + 255) / 256));
+  BY_T(f32,
+       hipLaunchKernelGGL(softcap_kernel<u16>, g, dim3(256), 0, st, (const u16*)x, cap, y, n),
+       hipLaunchKernelGGL(softcap_kernel<float>, g, dim3(256), 0, st, (const float*)x, cap, y, n))
+  return (int)hipGetLastError();
+}
+
+extern "C" int dllm_gated_group_norm(const float* y, const void* z, long ldz, int f32, const float* w, void* out, int rows,
+                                     int n, int groups, float eps, hipStream_t st) {
+  if (rows <= 0) return 0;
+  if (groups < 1 || n % groups) return -1;
+  const dim3 g((rows * groups + 3) / 4);
+  BY_T(f32,
+       hipLaunchKernelGGL(gated_group_norm_kernel<u16>, g, dim3(256), 0, st, y, (const u16*)z, ldz, w, (u16*)out, rows, n / groups, groups, eps),
+       hipLaunchKernelGGL(gated_group_norm_kernel<float>, g, dim3(256), 0, st, y, (const float*)z, ldz, w, (float*)out, rows, n / groups, groups, eps))
   return (int)hipGetLastError();
 }

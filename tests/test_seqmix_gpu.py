@@ -350,3 +350,137 @@ def test_delta_rule_and_conv_refill(dt, case, H, G, d, dv, K):
         ref.conv_state_refill(proj, c1, qstart, qlen, ctx, rows)
         torch.testing.assert_close(y1.float(), y2.float(), **tol(dt))
         torch.testing.assert_close(c3.float(), c1.float(), atol=0, rtol=0)
+
+
+# ----------------------------------------------------------------------------- differential attention, Mamba-2, mLSTM, PolyNorm, grouped router
+
+@pytest.mark.parametrize("dt", DTYPES)
+@pytest.mark.parametrize("n,groups", [(24, 1), (96, 4), (328, 2), (1000, 5), (66, 33)])
+def test_group_norms(dt, n, groups):
+    torch.manual_seed(9)
+    x = torch.randn(11, n + 8, device=DEV).to(dt)[:, 3:3 + n]
+    w = torch.randn(n, device=DEV)
+    torch.testing.assert_close(seqmix.rms_rows(x, w, 1e-6, groups=groups).float(),
+                               ref.rms_rows(x, w, 1e-6, groups=groups).float(), **tol(dt))
+    y, bias = torch.randn(11, n, device=DEV).to(dt), torch.randn(n, device=DEV)
+    for b in (None, bias):
+        r1 = torch.randn(11, n, device=DEV)
+        r2 = r1.clone()
+        l1 = torch.empty(11, n, device=DEV, dtype=dt)
+        l2 = l1.clone()
+        seqmix.norm_resadd(y, w, 1e-6, r1, l1, groups=groups, bias=b)
+        ref.norm_resadd(y, w, 1e-6, r2, l2, groups=groups, bias=b)
+        torch.testing.assert_close(r1, r2, atol=1e-5, rtol=1e-5)
+        torch.testing.assert_close(l1.float(), l2.float(), **tol(dt))
+    yy, z = torch.randn(11, n, device=DEV), torch.randn(11, n + 5, device=DEV).to(dt)
+    torch.testing.assert_close(seqmix.gated_group_norm(yy, z, w, groups, 1e-6, dt).float(),
+                               ref.gated_group_norm(yy, z, w, groups, 1e-6, dt).float(), **tol(dt))
+
+
+@pytest.mark.parametrize("dt", DTYPES)
+@pytest.mark.parametrize("case", CASES + [([40, 3], [90, 130])])
+@pytest.mark.parametrize("H,G,d,dv,rot,win", [(4, 2, 16, 8, 8, 5), (6, 2, 88, 56, 20, 64), (3, 3, 40, 72, 40, 1), (8, 1, 64, 64, 32, 100),
+                                              (4, 1, 56, 88, 28, 70), (2, 1, 136, 200, 64, 0), (5, 5, 24, 40, 0, 17)])
+def test_diff_attention_kernels(dt, case, H, G, d, dv, rot, win):
+    """Prep (bias, weighted norm before rotation, two maps a head), windowed attention with shared
+    values in both kernel forms and every split count, and the combination of the maps."""
+    from distributed_llm_amd.models.llama import AttnMeta
+    torch.manual_seed(14)
+    T, qstart, qlen, ctx, pos, bt, kc, _, slots = _pages(case, 2 * G, d, dv, dt)
+    vc = torch.randn(kc.shape[0], G, dv, 16, device=DEV).to(dt)
+    cols = 2 * H * d + 2 * G * d + G * dv
+    proj = torch.randn(T, cols + 3, device=DEV).to(dt)
+    bias = torch.randn(cols, device=DEV) * 0.3
+    qw, kw = torch.rand(d, device=DEV) + 0.5, torch.rand(d, device=DEV) + 0.5
+    table = ops.rope_cos_sin(256, max(rot, 2), 100.0, DEV)
+    kc2, vc2 = kc.clone(), vc.clone()
+    q1 = seqmix.qk_norm_prep(proj, bias, H, G, 2, d, dv, qw, kw, table, rot, 1e-5, 0.3, pos, slots, kc, vc)
+    q2 = ref.qk_norm_prep(proj, bias, H, G, 2, d, dv, qw, kw, table, rot, 1e-5, 0.3, pos, slots, kc2, vc2)
+    torch.testing.assert_close(q1.float(), q2.float(), **tol(dt))
+    torch.testing.assert_close(kc.float(), kc2.float(), **tol(dt))
+    torch.testing.assert_close(vc.float(), vc2.float(), **tol(dt))
+    q3 = seqmix.qk_norm_prep(proj, bias[:2 * H * d], H, G, 2, d, dv, qw, kw, table, rot, 1e-5, 0.3, pos, slots, None, None)
+    torch.testing.assert_close(q3.float(), q2.float(), **tol(dt))       # a layer that reads another layer's pages
+    want = ref.paged_gqa_attention(q2, kc2, vc2, bt, qstart, qlen, ctx, None, win, True)
+    meta = AttnMeta(slots=None, block_tables=bt, qstart=qstart, qlen=qlen, ctx=ctx, tile_seq=None, tile_tok0=None,
+                    last_idx=None, host_qlen=case[0])
+    forms = [False] + ([True] if seqmix.gqa_use_mfma(q2, 2 * H, 2 * G, d, dv, 16) else [])
+    for mfma in forms:
+        ts, tt = meta.latent_tiles(1, DEV, seqmix.gqa_tokens_per_tile(2 * H, 2 * G, mfma))
+        for splits in ((1, 2, 7) if mfma else (1,)):
+            got = seqmix.paged_gqa_attention(q2, kc2, vc2, bt, qstart, qlen, ctx, ts, tt, None, mfma, splits, window=win,
+                                             out_f32=True)
+            assert got.dtype == torch.float32
+            torch.testing.assert_close(got, want, **tol(dt))
+    o1 = seqmix.diff_combine(want, H, G, dv, 0.37, 1e-5, 0.7, dt)
+    o2 = ref.diff_combine(want, H, G, dv, 0.37, 1e-5, 0.7, dt)
+    torch.testing.assert_close(o1.float(), o2.float(), **tol(dt))
+
+
+@pytest.mark.parametrize("dt", DTYPES)
+@pytest.mark.parametrize("case", CASES)
+@pytest.mark.parametrize("H,dv,N,G", [(4, 32, 24, 2), (3, 40, 20, 3), (2, 8, 128, 1), (6, 70, 5, 2), (1, 64, 300, 1)])
+def test_ssd_scan(dt, case, H, dv, N, G):
+    torch.manual_seed(15)
+    qlens, starts = case
+    T, qstart, qlen, ctx, rows, _ = batch(qlens, starts)
+    slots = len(qlens) + 1
+    inner = H * dv
+    xbc = torch.randn(T, inner + 2 * G * N, device=DEV).to(dt)
+    proj = torch.randn(T, 2 * inner + 2 * G * N + H + 3, device=DEV).to(dt)
+    dt_col = 2 * inner + 2 * G * N
+    dt_b, neg_a, D = torch.randn(H, device=DEV), -torch.rand(H, device=DEV) * 2, torch.randn(H, device=DEV)
+    s1 = torch.randn(slots, H, N, dv, device=DEV)
+    s2 = s1.clone()
+    y1 = seqmix.ssd_scan(xbc, proj, dt_col, H, dv, N, G, dt_b, neg_a, D, s1, qstart, qlen, ctx, rows)
+    y2 = ref.ssd_scan(xbc, proj, dt_col, H, dv, N, G, dt_b, neg_a, D, s2, qstart, qlen, ctx, rows)
+    torch.testing.assert_close(y1, y2, atol=2e-3, rtol=2e-4)
+    torch.testing.assert_close(s1, s2, atol=2e-4, rtol=2e-4)
+
+
+@pytest.mark.parametrize("dt", DTYPES)
+@pytest.mark.parametrize("case", CASES)
+@pytest.mark.parametrize("H,d,dv", [(4, 40, 48), (3, 20, 40), (2, 128, 8), (1, 7, 70), (2, 200, 64)])
+def test_mlstm(dt, case, H, d, dv):
+    torch.manual_seed(16)
+    qlens, starts = case
+    T, qstart, qlen, ctx, rows, _ = batch(qlens, starts)
+    slots = len(qlens) + 1
+    proj = torch.randn(T, 2 * H * (d + dv + 1) + 5, device=DEV).to(dt)
+    proj[:, 2 * H * (d + dv):] *= 4          # gate logits across the cap's bend
+    gate_b = torch.randn(2 * H, device=DEV)
+    w = torch.rand(H * dv, device=DEV) + 0.5
+    s1 = torch.randn(slots, H, d, dv, device=DEV)
+    nm1 = torch.randn(slots, H, 1, d + 1, device=DEV).repeat(1, 1, seqmix.scan_col_blocks(dv), 1).contiguous()
+    s2, nm2 = s1.clone(), nm1.clone()
+    o1 = seqmix.mlstm(proj, H, d, dv, gate_b, 3.0, s1, nm1, 1e-5, w, qstart, qlen, ctx, rows)
+    o2 = ref.mlstm(proj, H, d, dv, gate_b, 3.0, s2, nm2, 1e-5, w, qstart, qlen, ctx, rows)
+    torch.testing.assert_close(o1.float(), o2.float(), **(tol(dt) if dt == torch.bfloat16 else dict(atol=2e-4, rtol=2e-4)))
+    torch.testing.assert_close(s1, s2, atol=2e-4, rtol=2e-4)
+    torch.testing.assert_close(nm1, nm2, atol=2e-4, rtol=2e-4)
+
+
+@pytest.mark.parametrize("dt", DTYPES)
+def test_polynorm_swiglu_softcap(dt):
+    torch.manual_seed(17)
+    for n in (24, 344, 1000):
+        z = (torch.randn(9, n + 4, device=DEV) * 2).to(dt)[:, 1:1 + n]
+        coef = torch.tensor([0.7, -0.4, 0.2, 0.1], device=DEV)
+        torch.testing.assert_close(seqmix.polynorm(z, coef, 1e-6).float(), ref.polynorm(z, coef, 1e-6).float(), **tol(dt))
+    E, ff = 6, 20
+    gu = torch.randn(9, E * 2 * ff, device=DEV).to(dt)
+    gate = torch.rand(9, E, device=DEV) * (torch.rand(9, E, device=DEV) > 0.5)
+    torch.testing.assert_close(seqmix.swiglu_scale(gu, gate, ff).float(), ref.swiglu_scale(gu, gate, ff).float(), **tol(dt))
+    x = (torch.randn(9, 77, device=DEV) * 40).to(dt)
+    torch.testing.assert_close(seqmix.softcap(x, 25.0), ref.softcap(x, 25.0), atol=1e-4, rtol=1e-5)
+
+
+@pytest.mark.parametrize("E,top,count,keep", [(16, 3, 2, 1), (16, 4, 1, 1), (12, 3, 4, 2), (64, 8, 8, 3), (5, 5, 5, 5), (6, 1, 6, 1),
+                                              (200, 6, 4, 4)])
+def test_group_router(E, top, count, keep):
+    torch.manual_seed(18)
+    logits = torch.randn(37, E, device=DEV) * 2
+    i1, w1 = seqmix.group_router(logits, top, count, keep)
+    i2, w2 = ref.group_router(logits, top, count, keep)
+    assert torch.equal(i1, i2)
+    torch.testing.assert_close(w1, w2, atol=1e-6, rtol=1e-6)
