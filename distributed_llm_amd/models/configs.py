@@ -250,7 +250,7 @@ class HybridConfig:
                 f = L.mlp
                 n += H + f.experts * (H + (3 if f.act == "swiglu" else 2) * f.ff * H) + 2 * f.shared_ff * H
             elif isinstance(L.mlp, DenseSpec):
-                n += 2 * H + 2 * L.mlp.ff * H + (4 if L.mlp.act == "polynorm" else 0)
+                n += (2 if self.pre_norm else 1) * H + 2 * L.mlp.ff * H + (4 if L.mlp.act == "polynorm" else 0)
         if self.depth_average:
             n += sum(i + 2 for i in range(len(self.layers)))
         return n

@@ -89,7 +89,7 @@ def diff_attention(h, W, p, m, eps, kv):
     lam = (torch.exp((W[p + "lq1"] * W[p + "lk1"]).sum()) - torch.exp((W[p + "lq2"] * W[p + "lk2"]).sum())
            + m["diff"])
     i, j = torch.arange(T)[:, None], torch.arange(T)[None, :]
-    seen = (i - j >= 0) & (i - j < m["mask"]["size"])
+    seen = (i - j >= 0) & (i - j < m["mask"]["size"]) if m.get("mask") else i - j >= 0
     out = torch.zeros(T, H, dv, dtype=F64)
     for hh in range(H):
         g = hh // (H // G)
@@ -160,7 +160,8 @@ def dense_ff(h, W, p, eps):
 def route(h, W, p, r):
     """Sigmoid scores; a group of neighbouring experts scores the sum of its two best; the ``top``
     best experts of the ``keep`` best groups, weights = their scores.  Returns [T, experts]."""
-    E, top, cnt, keep = r["experts"], r["top"], r["groups"]["count"], r["groups"]["keep"]
+    g = r.get("groups") or {"count": 1, "keep": 1}
+    E, top, cnt, keep = r["experts"], r["top"], g["count"], g["keep"]
     s = torch.sigmoid(h @ W[p + "router"].T)
     T = s.shape[0]
     gs = s.view(T, cnt, E // cnt).topk(min(2, E // cnt), -1).values.sum(-1)
@@ -213,3 +214,12 @@ def forward(cfg, W, tokens, taps=None):
     lg = group_norm(x, W["final.norm"], groups, eps) @ W["head"].T
     cap = cfg.get("logit_softcap")
     return cap * torch.tanh(lg / cap) if cap else lg
+
+
+def greedy(cfg, W, prompt, n):
+    """n arg-max continuations of a prompt (the whole sequence is recomputed for every token)."""
+    seq, out = list(prompt), []
+    for _ in range(n):
+        out.append(int(forward(cfg, W, seq)[-1].argmax()))
+        seq.append(out[-1])
+    return out
