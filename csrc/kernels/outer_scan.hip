@@ -11,7 +11,7 @@
 //              y = S^T q / (max(|n . q|, exp(-m')) + 1e-6).  mlstm_finish: heads to unit RMS, weight,
 //              sigmoid gate.
 //
-// One workgroup per (32 value columns, head, sequence); thread = (column, strip of state rows): a
+// One workgroup per (16 value columns, head, sequence); thread = (column, strip of state rows): a
 // thread keeps rows strip, strip + strips, ... of its column in registers.  Tokens run in groups of
 // 16: the group's k / q rows, values and gate numbers are staged once in LDS, every thread then walks
 // the 16 tokens on its registers and leaves per-strip partial sums in LDS, and after one barrier
@@ -29,13 +29,15 @@ template <typename T> __device__ __forceinline__ void stf(T* p, float v);
 template <> __device__ __forceinline__ void stf<u16>(u16* p, float v) { *p = f2bf(v); }
 template <> __device__ __forceinline__ void stf<float>(float* p, float v) { *p = v; }
 
-constexpr int OS_COLS = 32;   // value columns per workgroup
+constexpr int OS_COLS = 16;   // value columns per workgroup
 constexpr int OS_TG = 16;     // tokens per group
 
 __device__ __forceinline__ float softplus_f(float x) { return x > 20.f ? x : log1pf(expf(x)); }
 __device__ __forceinline__ float logsigmoid_f(float x) { return x < 0.f ? x - log1pf(expf(x)) : -log1pf(expf(-x)); }
 
-// MLSTM = false: ssd_scan; true: mlstm.  NPT >= ceil(N / strips).
+// MLSTM = false: ssd_scan; true: mlstm.  NPT >= ceil(N / strips); the staged k / q rows are padded with
+// zeros to NPT * strips entries, so the walk over a thread's state rows has no bounds test (rows past
+// N stay zero) and its LDS reads (k and q of a row side by side, 8 bytes) can be issued together.
 template <typename T, bool MLSTM, int NPT>
 __global__ void __launch_bounds__(256) outer_scan_kernel(const T* __restrict__ kq, long ld_kq, int k_off, int q_off, int kq_heads_div,
                                                          const T* __restrict__ vsrc, long ld_v, int v_off,
@@ -60,9 +62,9 @@ __global__ void __launch_bounds__(256) outer_scan_kernel(const T* __restrict__ k
   const int v0 = cb * OS_COLS;
   const bool is_norm = MLSTM && c == OS_COLS;
   const bool col_ok = live && (is_norm || v0 + c < dv);
-  float* Ks = sm;                       // [TG][N]
-  float* Qs = Ks + OS_TG * N;           // [TG][N]
-  float* Vs = Qs + OS_TG * N;           // [TG][CW]
+  constexpr int NP = NPT * STRIPS;
+  float2* KQ = reinterpret_cast<float2*>(sm);   // [TG][NP] (k, q)
+  float* Vs = sm + 2 * OS_TG * NP;      // [TG][CW]
   float* Ga = Vs + OS_TG * CW;          // [TG]  SSD: a_t;  mLSTM: i_t
   float* Gb = Ga + OS_TG;               // [TG]  SSD: b_t;  mLSTM: f_t
   float* Ms = Gb + OS_TG;               // [TG]  mLSTM: m_t
@@ -84,11 +86,14 @@ __global__ void __launch_bounds__(256) outer_scan_kernel(const T* __restrict__ k
   for (int t0 = 0; t0 < n_new; t0 += OS_TG) {
     const int nt = min(OS_TG, n_new - t0);
     __syncthreads();     // the previous group's sums are stored
-    for (int e = tid; e < nt * N; e += 256) {
-      const int t = e / N, n = e % N;
-      const T* r = kq + (long)(q0 + t0 + t) * ld_kq + (long)kh * N + n;
-      Ks[e] = ldf(r + k_off);
-      Qs[e] = ldf(r + q_off) * qscale;
+    for (int e = tid; e < nt * NP; e += 256) {
+      const int t = e / NP, n = e % NP;
+      float2 v = make_float2(0.f, 0.f);
+      if (n < N) {
+        const T* r = kq + (long)(q0 + t0 + t) * ld_kq + (long)kh * N + n;
+        v = make_float2(ldf(r + k_off), ldf(r + q_off) * qscale);
+      }
+      KQ[e] = v;
     }
     for (int e = tid; e < nt * CW; e += 256) {
       const int t = e / CW, cc = e % CW;
@@ -126,16 +131,13 @@ __global__ void __launch_bounds__(256) outer_scan_kernel(const T* __restrict__ k
           b = Gb[t];
         }
         const float bv = b * Vs[t * CW + c];
-        const float* kr = Ks + t * N;
-        const float* qr = Qs + t * N;
+        const float2* kqr = KQ + t * NP + strip;
         float acc = 0.f;
 #pragma unroll
         for (int k = 0; k < NPT; ++k) {
-          const int n = strip + k * STRIPS;
-          if (n < N) {
-            S[k] = a * S[k] + kr[n] * bv;
-            acc += S[k] * qr[n];
-          }
+          const float2 kq2 = kqr[k * STRIPS];
+          S[k] = a * S[k] + kq2.x * bv;
+          acc += S[k] * kq2.y;
         }
         Ps[(t * STRIPS + strip) * CW + c] = acc;
       }
@@ -190,10 +192,22 @@ __global__ void __launch_bounds__(256) head_norm_gate_kernel(const float* __rest
   }
 }
 
+constexpr int OS_NPT[] = {1, 2, 3, 4, 5, 6, 8, 9, 10, 12, 16, 20, 24, 32};   // instantiated rows per thread
+
+template <bool MLSTM> int outer_npt(int N) {
+  constexpr int STRIPS = 256 / (OS_COLS + (MLSTM ? 1 : 0));
+  const int need = (N + STRIPS - 1) / STRIPS;
+  for (int v : OS_NPT)
+    if (v >= need) return v;
+  return -1;
+}
+
 template <bool MLSTM> long outer_lds(int N) {
   constexpr int CW = OS_COLS + (MLSTM ? 1 : 0);
   constexpr int STRIPS = 256 / CW;
-  return 4L * (2L * OS_TG * N + OS_TG * CW + 3 * OS_TG + (long)OS_TG * STRIPS * CW);
+  const int npt = outer_npt<MLSTM>(N);
+  if (npt < 0) return 1L << 40;
+  return 4L * (2L * OS_TG * npt * STRIPS + OS_TG * CW + 3 * OS_TG + (long)OS_TG * STRIPS * CW);
 }
 
 #define ENSURE_LDS(kernel, bytes)                                                                                \
@@ -219,15 +233,13 @@ int launch_outer(dim3 grid, long lds, hipStream_t st, const void* kq, long ld_kq
 
 template <typename T, bool MLSTM, typename... A>
 int launch_outer_npt(int N, A... a) {
-  constexpr int STRIPS = 256 / (OS_COLS + (MLSTM ? 1 : 0));
-  const int npt = (N + STRIPS - 1) / STRIPS;
-  if (npt <= 2) return launch_outer<T, MLSTM, 2>(a...);
-  if (npt <= 4) return launch_outer<T, MLSTM, 4>(a...);
-  if (npt <= 8) return launch_outer<T, MLSTM, 8>(a...);
-  if (npt <= 16) return launch_outer<T, MLSTM, 16>(a...);
-  if (npt <= 32) return launch_outer<T, MLSTM, 32>(a...);
-  if (npt <= 64) return launch_outer<T, MLSTM, 64>(a...);
-  return -2;
+  switch (outer_npt<MLSTM>(N)) {
+#define OS_CASE(V) case V: return launch_outer<T, MLSTM, V>(a...);
+    OS_CASE(1) OS_CASE(2) OS_CASE(3) OS_CASE(4) OS_CASE(5) OS_CASE(6) OS_CASE(8) OS_CASE(9) OS_CASE(10) OS_CASE(12)
+    OS_CASE(16) OS_CASE(20) OS_CASE(24) OS_CASE(32)
+#undef OS_CASE
+    default: return -2;
+  }
 }
 
 }  // namespace

@@ -1,8 +1,8 @@
-"""Layer-list (Filevik, Sedopel) models beside the closest Llama-family model at equal size: prefill
-and decode throughput through the engine, and the time of each mixer kernel against its roofline.
+"""Layer-list (Filevik, Sedopel, Pebodra) models beside the closest Llama-family model at equal size:
+prefill and decode throughput through the engine, and the time of each mixer kernel against its roofline.
 
-``python bench.py --arch-bench [--arch-design filevik|sedopel] [--arch-size s|m]`` (random weights,
-synthetic tokens).  The default bench workload and its JSON line are untouched; this prints one
+``python bench.py --arch-bench [--arch-design filevik|sedopel|pebodra] [--arch-size s|m]`` (random
+weights, synthetic tokens).  The default bench workload and its JSON line are untouched; this prints one
 JSON object of its own.
 
 The Sedopel stack alternates parallel layers (grouped-query softmax attention beside lightning
@@ -11,6 +11,13 @@ comparison model is a dense Llama (grouped-query attention + SwiGLU of equal par
 the same width and depth, and kernel by kernel: paged attention against the Llama attention kernels
 at the same head counts, lightning attention against retention, the delta rule against the
 selective scan.
+
+The Pebodra stack cycles differential sliding-window attention -> mLSTM -> attention on the first
+layer's keys and values -> Mamba-2, the first layer with a dense PolyNorm feed-forward and the
+others with group-routed SwiGLU experts; its comparison model is the Mixtral-style Llama of the same
+width, depth and experts, and kernel by kernel: windowed attention with two maps a head against the
+Sedopel attention kernel (the same kernel without a window) and the Llama kernels at the same
+number of score rows, Mamba-2 against the selective scan and the delta rule, mLSTM against retention.
 
 Sizes: width / layers of a small and a mid-size decoder.  The Filevik stack cycles mamba1 ->
 retention -> latent attention, each with routed squared-ReLU experts and a shared expert; the
@@ -45,6 +52,125 @@ SEDOPEL_SIZES = {
     "m": dict(width=2048, layers=12, heads=32, kv_heads=8, dim=64, vdim=64, rot=32, l_heads=16, l_dim=128, l_vdim=128,
               d_heads=16, d_kv_heads=8, d_dim=128, d_vdim=128, conv=4, ff=8192, vocab=32000),
 }
+
+
+PEBODRA_SIZES = {
+    "s": dict(width=1024, layers=6, heads=8, kv_heads=2, dim=64, vdim=128, rot=64, window=1024, m_heads=32, m_vdim=64,
+              state=128, groups=4, conv=4, norm_groups=8, x_heads=8, x_dim=64, x_vdim=128, experts=8, top=2, ff=1024,
+              dense_ff=4096, vocab=32000),
+    "m": dict(width=2048, layers=12, heads=16, kv_heads=4, dim=64, vdim=128, rot=64, window=1024, m_heads=64, m_vdim=64,
+              state=128, groups=8, conv=4, norm_groups=8, x_heads=16, x_dim=128, x_vdim=128, experts=8, top=2, ff=2048,
+              dense_ff=8192, vocab=32000),
+}
+
+
+def pebodra_raw(z: dict) -> dict:
+    moe = {"kind": "moe", "expert": {"ff": z["ff"]},
+           "router": {"experts": z["experts"], "top": z["top"], "groups": {"count": 2, "keep": 1}}}
+    att = {"heads": z["heads"], "kv_heads": z["kv_heads"], "dim": z["dim"], "vdim": z["vdim"], "diff": 0.2,
+           "scale": z["dim"] ** -0.5, "mask": {"size": z["window"]}, "rot": {"dims": z["rot"], "base": 10000.0}}
+    layers = []
+    for i in range(z["layers"]):
+        k = i % 4
+        if k == 0:
+            L = {"type": "attention", "mixer": dict(att)}
+        elif k == 2:
+            L = {"type": "attention", "mixer": dict(att, kv_from=i - 2)}
+        elif k == 1:
+            L = {"type": "mlstm", "mixer": {"heads": z["x_heads"], "dim": z["x_dim"], "vdim": z["x_vdim"], "gate_cap": 10.0}}
+        else:
+            L = {"type": "mamba2", "mixer": {"heads": z["m_heads"], "vdim": z["m_vdim"], "state": z["state"],
+                                             "groups": z["groups"], "conv": z["conv"], "norm_groups": z["norm_groups"]}}
+        L["mlp"] = {"kind": "dense", "ff": z["dense_ff"]} if i == 0 else moe
+        layers.append(L)
+    return {"architecture": "Pebodra", "width": z["width"], "vocab": z["vocab"], "norm": {"eps": 1e-6, "groups": 4},
+            "logit_softcap": 50.0, "layers": layers}
+
+
+def pebodra_twin(z: dict):
+    """Mixtral-style Llama of the same width, depth, vocabulary, expert count / top-k and expert width
+    (both run SwiGLU experts)."""
+    from ..models.configs import ModelConfig
+    return ModelConfig(f"moe-llama-{z['width']}", z["width"], z["layers"], z["width"] // 64, max(1, z["width"] // 256), 64,
+                       z["ff"], z["vocab"], 10000.0, 1e-6, 16384, n_experts=z["experts"], experts_per_token=z["top"])
+
+
+def pebodra_kernel_rooflines(z: dict, T: int = 4096, B: int = 64, ctx: int = 2048) -> Dict[str, dict]:
+    """Each Pebodra mixer kernel alone (bf16): prefill of one T-token sequence, decode of B sequences
+    at ``ctx``; time, the bound resource's minimum time, and their ratio."""
+    from .. import ops
+    from ..models.llama import AttnMeta
+    from ..ops import seqmix
+    dev, bf = "cuda", torch.bfloat16
+    i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=dev)
+    res: Dict[str, dict] = {}
+
+    def rec(name, sec, bytes_, flops, peak_flops):
+        floor = max(bytes_ / PEAK_BW, flops / peak_flops)
+        res[name] = {"us": round(sec * 1e6, 1), "roofline_us": round(floor * 1e6, 2), "x_roofline": round(sec / floor, 1),
+                     "bound": "memory" if bytes_ / PEAK_BW >= flops / peak_flops else "compute"}
+
+    for tag, qlens, starts in (("prefill", [T], [0]), ("decode", [1] * B, [ctx] * B)):
+        n, S = sum(qlens), len(qlens)
+        qstart = i32([sum(qlens[:i]) for i in range(S)])
+        cxl = [a + b for a, b in zip(starts, qlens)]
+        qlen, cx, rows = i32(qlens), i32(cxl), i32(list(range(S)))
+        pos = i32([p for a, m in zip(starts, qlens) for p in range(a, a + m)])
+        # differential attention: prep, windowed attention over both maps, combination
+        H, G, d, dv, Wn = z["heads"], z["kv_heads"], z["dim"], z["vdim"], z["window"]
+        pairs = sum(min(p + 1, Wn) for a, m in zip(starts, qlens) for p in range(a, a + m))   # (query, visible key) pairs
+        seen = sum(min(c, Wn + m - 1) for c, m in zip(cxl, qlens))                            # keys any row of a sequence sees
+        nb = (max(cxl) + 15) // 16
+        bt = torch.arange(S * nb, dtype=torch.int32, device=dev).view(S, nb)
+        kc = (torch.randn(S * nb, 2 * G, 16, d, device=dev) * 0.3).to(bf)
+        vc = (torch.randn(S * nb, G, dv, 16, device=dev) * 0.3).to(bf)
+        cols = 2 * H * d + 2 * G * d + G * dv
+        proj, bias = torch.randn(n, cols, device=dev).to(bf), torch.zeros(cols, device=dev)
+        table = ops.rope_cos_sin(ctx + T + 8, z["rot"], 10000.0, dev)
+        slots = i32([int(bt[i, p // 16]) * 16 + p % 16 for i, (a, m) in enumerate(zip(starts, qlens)) for p in range(a, a + m)])
+        nw = torch.ones(d, device=dev)
+        prep = lambda: seqmix.qk_norm_prep(proj, bias, H, G, 2, d, dv, nw, nw, table, z["rot"], 1e-6, d ** -0.5, pos, slots, kc, vc)
+        q = prep()
+        rec(f"qk_prep_{tag}", _timed(prep), n * cols * 4 + n * 2 * H * d * 2, n * 2 * (H + G) * d * 10, PEAK_F32)
+        meta = AttnMeta(slots=None, block_tables=bt, qstart=qstart, qlen=qlen, ctx=cx, tile_seq=None, tile_tok0=None,
+                        last_idx=None, host_qlen=qlens)
+        mfma = seqmix.gqa_use_mfma(q, 2 * H, 2 * G, d, dv, 16)
+        ts, tt = meta.latent_tiles(1, dev, seqmix.gqa_tokens_per_tile(2 * H, 2 * G, mfma))
+        sp = seqmix.gqa_splits(int(ts.numel()), 2 * G, max(cxl), Wn) if mfma else 1
+        att = lambda: seqmix.paged_gqa_attention(q, kc, vc, bt, qstart, qlen, cx, ts, tt, None, mfma, sp, window=Wn, out_f32=True)
+        a = att()
+        rec(f"attention_{tag}", _timed(att, 3), seen * G * (2 * d + dv) * 2 + n * 2 * H * (d * 2 + dv * 4),
+            pairs * 2 * H * 2 * (d + dv), PEAK_BF16)
+        rec(f"diff_combine_{tag}", _timed(lambda: seqmix.diff_combine(a, H, G, dv, 0.2, 1e-6, 0.8, bf)),
+            n * H * dv * (8 + 2), n * H * dv * 6, PEAK_F32)
+        # Mamba-2: convolution, recurrence, gated norm
+        Hm, dvm, N, Gm, K = z["m_heads"], z["m_vdim"], z["state"], z["groups"], z["conv"]
+        inner, C = Hm * dvm, Hm * dvm + 2 * Gm * N
+        pr = torch.randn(n, 2 * inner + 2 * Gm * N + Hm, device=dev).to(bf)
+        conv_s, st = torch.zeros(S, K - 1, C, device=dev, dtype=bf), torch.zeros(S, Hm, N, dvm, device=dev)
+        w, b_ = torch.randn(C, K, device=dev) * 0.5, torch.zeros(C, device=dev)
+        xin = pr[:, inner:]
+        xbc = seqmix.causal_conv_silu(xin, w, b_, conv_s, qstart, qlen, cx, rows)
+        dtb, na, D = torch.zeros(Hm, device=dev), -torch.rand(Hm, device=dev), torch.ones(Hm, device=dev)
+        rec(f"ssd_conv_{tag}", _timed(lambda: seqmix.causal_conv_silu(xin, w, b_, conv_s, qstart, qlen, cx, rows)),
+            n * C * 4 + (S * (K - 1) * C * 2 if tag == "decode" else 0), n * C * 2 * K, PEAK_F32)
+        scan = lambda: seqmix.ssd_scan(xbc, pr, 2 * inner + 2 * Gm * N, Hm, dvm, N, Gm, dtb, na, D, st, qstart, qlen, cx, rows)
+        y = scan()
+        rec(f"ssd_scan_{tag}", _timed(scan), n * (C * 2 + inner * 4) + (S * Hm * N * dvm * 8 if tag == "decode" else 0),
+            n * Hm * N * dvm * 4, PEAK_F32)
+        gw = torch.ones(inner, device=dev)
+        rec(f"gated_norm_{tag}", _timed(lambda: seqmix.gated_group_norm(y, pr, gw, z["norm_groups"], 1e-6, bf)),
+            n * inner * (4 + 2 + 2), n * inner * 8, PEAK_F32)
+        # mLSTM
+        Hx, dx, dvx = z["x_heads"], z["x_dim"], z["x_vdim"]
+        px = torch.randn(n, 2 * Hx * (dx + dvx + 1), device=dev).to(bf)
+        sx = torch.zeros(S, Hx, dx, dvx, device=dev)
+        nm = torch.zeros(S, Hx, seqmix.scan_col_blocks(dvx), dx + 1, device=dev)
+        gb, hw = torch.zeros(2 * Hx, device=dev), torch.ones(Hx * dvx, device=dev)
+        rec(f"mlstm_{tag}", _timed(lambda: seqmix.mlstm(px, Hx, dx, dvx, gb, 10.0, sx, nm, 1e-6, hw, qstart, qlen, cx, rows)),
+            n * (2 * Hx * dx + 3 * Hx * dvx) * 2 + (S * Hx * dx * dvx * 8 if tag == "decode" else 0),
+            n * Hx * dx * (dvx + 1) * 4, PEAK_F32)
+    return res
 
 
 def sedopel_raw(z: dict) -> dict:
@@ -306,7 +432,24 @@ def llama_kernel_rooflines(T: int = 4096, B: int = 64, ctx: int = 2048, nq: int 
 
 
 def run(size: str = "s", kernels_only: bool = False, design: str = "filevik") -> dict:
-    from ..models.configs import filevik_config, sedopel_config
+    from ..models.configs import filevik_config, pebodra_config, sedopel_config
+    if design == "pebodra":
+        z = PEBODRA_SIZES[size]
+        out = {"bench": "arch", "design": design, "size": size, "dtype": "bf16", "data": "synthetic", "sizes": z}
+        out["pebodra_kernels"] = pebodra_kernel_rooflines(z)
+        # the like kernels at like sizes: the attention kernel without window and maps at the same
+        # number of score rows, the delta rule, lightning / retention, the selective scan
+        out["sedopel_kernels"] = sedopel_kernel_rooflines(dict(SEDOPEL_SIZES[size], heads=2 * z["heads"],
+                                                               kv_heads=2 * z["kv_heads"], dim=z["dim"], vdim=z["vdim"]))
+        out["filevik_kernels"] = kernel_rooflines(SIZES[size])
+        out["llama_kernels"] = llama_kernel_rooflines(nq=2 * z["heads"], nkv=2 * z["kv_heads"], d=z["dim"])
+        if not kernels_only:
+            prompts, batches = [512, 2048], [1, 16, 64]
+            out["pebodra"] = engine_throughput(pebodra_config(pebodra_raw(z), name=f"pebodra-{size}"), prompts, batches,
+                                               ctx=1024, new=32, rows=64)
+            out["moe_llama"] = engine_throughput(pebodra_twin(z), prompts, batches, ctx=1024, new=32, rows=64)
+        print(json.dumps(out))
+        return out
     if design == "sedopel":
         z = SEDOPEL_SIZES[size]
         out = {"bench": "arch", "design": design, "size": size, "dtype": "bf16", "data": "synthetic", "sizes": z}

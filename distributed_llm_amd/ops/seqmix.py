@@ -348,7 +348,7 @@ def diff_combine(a, heads, kv_heads, vdim, lam, eps, out_scale, out_dtype) -> to
 
 # ----------------------------------------------------------------------------- gated outer-product recurrences (Mamba-2, mLSTM)
 
-SCAN_COLS = 32      # value columns of one (sequence, head) a workgroup of the recurrence kernels owns
+SCAN_COLS = 16      # value columns of one (sequence, head) a workgroup of the recurrence kernels owns
 
 
 def scan_col_blocks(vdim: int) -> int:

@@ -45,7 +45,7 @@ def test_bench_json_line(n, extra, par, cfg):
     assert out["n_gpus"] == n and out["steps"] == 1 and out["warmup"] == 1
     assert out["value"] > 0 and out["higher_is_better"] is True
     assert out["scaling"] == ("weak" if cfg == 2 else "config")
-    assert out["per_gpu_tok_s"] * n == pytest.approx(out["value"], rel=1e-3)
+    assert out["per_gpu_tok_s"] * n == pytest.approx(out["value"], rel=1e-3, abs=0.011 * n)     # both are rounded to 0.01
     assert 0 < out["init_s"] <= out["startup_s"]
     assert out["config"]["parallelism"].startswith(par)
     if out["config"]["turn_pipelining"]:
