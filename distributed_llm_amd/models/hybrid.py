@@ -318,9 +318,14 @@ class HybridModel:
                 else:
                     w1 = torch.stack([t[p + f"mlp.e{e}.up"] for e in range(f.experts)])   # [E, ff, W]
                 w2 = torch.stack([t[p + f"mlp.e{e}.down"] for e in range(f.experts)])     # [E, W, ff]
-                D["w1"] = put(w1)
                 grouped = (dt == torch.bfloat16 and dev.type == "cuda" and W % 32 == 0 and f.ff % 32 == 0
                            and f.experts <= 64)
+                if f.act == "swiglu" and grouped and W % 64 == 0 and f.ff % 64 == 0:
+                    # the LDS-tiled grouped GEMM pairs gate and up rows in its epilogue: rows interleaved
+                    from .llama import gate_up_order
+                    w1 = w1.index_select(1, gate_up_order(f.ff))
+                    D["tg"] = True
+                D["w1"] = put(w1)
                 if grouped or dev.type != "cuda":
                     D["w2"] = put(w2)
                 else:   # dense form: one down projection over every expert's columns
@@ -558,6 +563,8 @@ class HybridModel:
         ids, w = seqmix.group_router(logits, f.top, f.group_count, f.group_keep)
         if f.scale != 1.0:
             w = w * f.scale
+        if L.get("tg"):
+            return ops.moe_ffn_tg(x if x.stride(1) == 1 else x.contiguous(), ids, w, L["w1"], L["w2"])
         if "w2" in L and (not x.is_cuda or seqmix.moe_ffn_relu2_ok(x, L["w1"])):
             return ops.moe_ffn(x, ids, w, L["w1"], L["w2"])
         if "w2d" not in L:
