@@ -176,6 +176,7 @@ SINGLE = {
     "dense-ff": [mlstm(mlp=dense(31))], "moe": [mamba(mlp=moe())], "moe-no-groups": [mamba(mlp=moe(experts=5, top=5, count=1, keep=1))],
     "moe-keep-all": [mamba(mlp=moe(experts=8, top=3, count=4, keep=4))], "moe-single-expert-groups": [mamba(mlp=moe(experts=4, top=2, count=4, keep=3))],
     "moe-top-one": [mlstm(mlp=moe(experts=9, top=1, count=3, keep=1, ff=32))],
+    "moe-many-experts": [mamba(mlp=moe(experts=72, top=3, count=9, keep=2, ff=4))],
 }
 
 
@@ -337,7 +338,7 @@ def test_window_edges(tmp_path, device, window):
 
 
 @pytest.mark.parametrize("device", DEVICES)
-@pytest.mark.parametrize("n", [15, 16, 17, 63, 64, 65, 130])
+@pytest.mark.parametrize("n", [15, 16, 17, 63, 64, 65, 130, 330])
 def test_attention_sharp_far_keys(tmp_path, device, n):
     """Query/key weights scaled so that the softmax is peaked: one key, often far back and on either
     side of a page (16) or key-tile (64) border, carries a row; prompt and decoded rows; the second
@@ -345,7 +346,7 @@ def test_attention_sharp_far_keys(tmp_path, device, n):
     cfg = make_cfg([attn(heads=2, kv_heads=1, dim=8, vdim=5, rot=4, scale=3.0, window=500),
                     attn(heads=2, kv_heads=1, dim=8, vdim=5, rot=4, scale=2.0, window=33, diff=0.5, kv_from=0)], width=16, groups=2)
     W = make_weights(cfg, seed=n, qk_gain=2.0)
-    eng = engine(write_model(tmp_path / "m", cfg, W), device, torch.float32)
+    eng = engine(write_model(tmp_path / "m", cfg, W), device, torch.float32, tokens=max(256, n + 32))
     t = toks(n + 2, seed=n)
     want = orc.forward(cfg, W, t)
     got = [eng.feed([("a", t[:n], list(range(n)))]), eng.feed([("a", t[n:n + 1], [0])]), eng.feed([("a", t[n + 1:], [0])], ["a"])]
