@@ -1,6 +1,10 @@
 """Sequence-mixer ops beside softmax attention: short causal convolution, selective scan, decayed
 linear attention (retention), latent attention over a shared compressed key/value, the f32
-residual update, squared-ReLU experts (csrc/kernels/seqmix.hip, latent.hip, moe.hip).
+residual update, squared-ReLU experts (csrc/kernels/seqmix.hip, latent.hip, moe.hip); grouped-query
+attention over pages with an optional window and shared value heads, its input kernels (unit-RMS or
+weighted q/k norms, one or two score maps a head) and the gated delta rule (gqa.hip, delta.hip); the
+Mamba-2 and mLSTM recurrences (outer_scan.hip); PolyNorm, the group-limited sigmoid router, the
+dense form of SwiGLU experts and the logit soft cap.
 
 Same dispatch rule as the rest of the op library: GPU tensors run the HIP kernel (or raise when the
 extension is missing), CPU tensors the torch reference.  Every kernel takes bf16 or f32 activations
