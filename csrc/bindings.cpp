@@ -51,6 +51,12 @@ int dllm_moe_ffn(const void*, long, long, int, const int*, const float*, int, in
 int dllm_rms_rows(const void*, long, int, const float*, void*, long, int, int, int, float, int, hipStream_t);
 int dllm_norm_resadd(const void*, long, int, const float*, float*, void*, int, int, float, int, const float*, hipStream_t);
 int dllm_polynorm(const void*, long, int, const float*, void*, long, int, float, hipStream_t);
+int dllm_route_topk(const float*, long, int, int, int, int, int, int, int, const float*, int, int*, float*, float*, hipStream_t);
+int dllm_ls_resadd_ln(const void*, long, int, const float*, const float*, const void*, long, const float*, long, const void*, long,
+                      const float*, float*, const float*, const float*, void*, long, int, float, hipStream_t);
+int dllm_glu_act(const void*, long, int, const float*, int, int, float, float, void*, long, hipStream_t);
+int dllm_proj_norm_prep(const void*, long, int, int, int, int, int, const float*, const float*, const float*, int, int, int, float,
+                        const float*, int, const int*, const int*, void*, void*, void*, long, int, hipStream_t);
 int dllm_group_router(const float*, int, int, int, int, int, int*, float*, hipStream_t);
 int dllm_swiglu_scale(const void*, int, const float*, int, int, void*, long, hipStream_t);
 int dllm_softcap(const void*, int, float, float*, long, hipStream_t);
@@ -64,7 +70,7 @@ int dllm_qk_norm_prep(const void*, long, int, const float*, int, int, int, int, 
                       int, int, float, float, const int*, const int*, void*, void*, void*, long, int, hipStream_t);
 int dllm_diff_combine(const float*, void*, int, long, int, int, int, float, float, float, hipStream_t);
 int dllm_conv_silu(const void*, long, int, const float*, const float*, void*, const int*, const int*, const int*,
-                   const int*, void*, int, int, int, int, int, hipStream_t);
+                   const int*, void*, int, int, int, int, int, int, hipStream_t);
 int dllm_selective_scan(const void*, const void*, int, const float*, const float*, const void*, long, int, const float*,
                         const void*, long, float*, void*, int, const int*, const int*, const int*, const int*, void*, int,
                         int, int, hipStream_t);
@@ -91,7 +97,7 @@ int dllm_gqa_tile_tokens(int, int, int);
 int dllm_gqa_mfma_ok(int, int, int, int, int, int);
 int dllm_paged_gqa(const void*, const void*, const void*, int, const int*, int, int, const int*, const int*, const int*,
                    const int*, const int*, int, const void*, long, void*, int, int, int, int, int, int, float*, int, int, int,
-                   hipStream_t);
+                   int, float, hipStream_t);
 int dllm_relu2_scale(const void*, int, const float*, int, int, void*, long, int, hipStream_t);
 int dllm_dense_gate(const int*, const float*, float*, long, int, int, hipStream_t);
 int dllm_latent_kv_write(const void*, long, int, int, int, const float*, float, const int*, const float*, int, const int*,
@@ -1382,8 +1388,9 @@ void norm_resadd(torch::Tensor y, torch::Tensor w, double eps, torch::Tensor x, 
 }
 
 void causal_conv_silu(torch::Tensor x, torch::Tensor w, torch::Tensor b, torch::Tensor state, torch::Tensor qstart,
-                      torch::Tensor qlen, torch::Tensor ctx, torch::Tensor rows, torch::Tensor y, bool refill) {
+                      torch::Tensor qlen, torch::Tensor ctx, torch::Tensor rows, torch::Tensor y, bool refill, int64_t act) {
   const bool f = act_f32(x, "x");
+  TORCH_CHECK(act == 0 || act == 1, "act: 0 (SiLU) or 1 (input plus convolution)");
   check_rows2d(x, "x");
   check_f32(w, "w");
   check_f32(b, "b");
@@ -1398,7 +1405,7 @@ void causal_conv_silu(torch::Tensor x, torch::Tensor w, torch::Tensor b, torch::
               "y [T, C]");
   auto m = seq_meta(qstart, qlen, ctx, rows, state.size(0));
   ok(dllm_conv_silu(x.data_ptr(), x.stride(0), f, w.data_ptr<float>(), b.data_ptr<float>(), state.data_ptr(), m.qstart,
-                    m.qlen, m.ctx, m.rows, y.data_ptr(), T, m.S, C, K, (int)refill, stream()),
+                    m.qlen, m.ctx, m.rows, y.data_ptr(), T, m.S, C, K, (int)refill, (int)act, stream()),
      "causal_conv_silu");
 }
 
@@ -1667,8 +1674,9 @@ void attn_prep(torch::Tensor proj, int64_t H, int64_t G, int64_t d, int64_t dv, 
 void paged_gqa_attention(torch::Tensor q, torch::Tensor kc, torch::Tensor vc, torch::Tensor bt, torch::Tensor qstart,
                          torch::Tensor qlen, torch::Tensor ctx, torch::Tensor tile_seq, torch::Tensor tile_tok0,
                          c10::optional<torch::Tensor> gate, torch::Tensor out, bool mfma, int64_t splits,
-                         c10::optional<torch::Tensor> part, int64_t window) {
+                         c10::optional<torch::Tensor> part, int64_t window, int64_t keep_first, double sink) {
   const bool f = act_f32(q, "q");
+  TORCH_CHECK(keep_first >= 0 && sink >= 0.0, "keep_first >= 0, sink >= 0");
   TORCH_CHECK(q.dim() == 3 && q.is_contiguous(), "q [T, H, d]");
   const int64_t T = q.size(0), H = q.size(1), d = q.size(2);
   for (auto* c : {&kc, &vc})
@@ -1712,7 +1720,7 @@ void paged_gqa_attention(torch::Tensor q, torch::Tensor kc, torch::Tensor vc, to
                                 (int)kc.size(2), qstart.data_ptr<int>(), qlen.data_ptr<int>(), ctx.data_ptr<int>(),
                                 tile_seq.data_ptr<int>(), tile_tok0.data_ptr<int>(), (int)tile_seq.numel(), gp, ldg,
                                 out.data_ptr(), (int)H, (int)G, (int)d, (int)dv, (int)mfma, (int)splits, pptr, (int)window,
-                                (int)GV, (int)of32, stream());
+                                (int)GV, (int)of32, (int)keep_first, (float)sink, stream());
   TORCH_CHECK(rc != -2, "head widths do not fit the LDS");
   ok(rc, "paged_gqa_attention");
 }
@@ -1885,6 +1893,147 @@ void swiglu_scale(torch::Tensor gu, torch::Tensor gate, int64_t ff, torch::Tenso
      "swiglu_scale");
 }
 
+void route_topk(torch::Tensor logits, int64_t E, int64_t top, int64_t count, int64_t keep, int64_t smode, int64_t gmode,
+                c10::optional<torch::Tensor> corr, int64_t real, torch::Tensor ids, torch::Tensor wts, torch::Tensor idw) {
+  check_f32(logits, "logits");
+  check_i32(ids, "ids");
+  check_f32(wts, "wts");
+  check_f32(idw, "idw");
+  TORCH_CHECK(logits.dim() == 2 && logits.stride(1) == 1 && logits.size(1) >= E, "logits [T, >= E], rows contiguous");
+  const int64_t T = logits.size(0);
+  TORCH_CHECK(E >= 1 && E <= 1024 && count >= 1 && E % count == 0 && keep >= 1 && keep <= count && top >= 1 &&
+                  top <= keep * (E / count) && real >= 0 && real <= E,
+              "outputs <= 1024, groups divide the outputs, top fits the kept groups");
+  TORCH_CHECK((smode == 0 || smode == 1) && (gmode == 0 || gmode == 1), "score / group score mode");
+  TORCH_CHECK(ids.is_contiguous() && wts.is_contiguous() && ids.numel() == T * top && wts.numel() == T * top &&
+                  idw.is_contiguous() && idw.numel() == T,
+              "ids / wts [T, top], idw [T]");
+  const float* cp = nullptr;
+  if (corr) {
+    check_f32(*corr, "correction");
+    TORCH_CHECK(corr->is_contiguous() && corr->numel() == E, "correction [E]");
+    cp = corr->data_ptr<float>();
+  }
+  ok(dllm_route_topk(logits.data_ptr<float>(), (long)logits.stride(0), (int)T, (int)E, (int)top, (int)count, (int)keep,
+                     (int)smode, (int)gmode, cp, (int)real, ids.data_ptr<int>(), wts.data_ptr<float>(), idw.data_ptr<float>(),
+                     stream()),
+     "route_topk");
+}
+
+void ls_resadd_ln(torch::Tensor x, torch::Tensor w, torch::Tensor b, double eps, torch::Tensor out,
+                  c10::optional<torch::Tensor> y, c10::optional<torch::Tensor> ls, c10::optional<torch::Tensor> bias,
+                  c10::optional<torch::Tensor> y2, c10::optional<torch::Tensor> g2, c10::optional<torch::Tensor> h,
+                  c10::optional<torch::Tensor> hw) {
+  check_f32(x, "x");
+  check_f32(w, "w");
+  check_f32(b, "b");
+  const bool f = act_f32(out, "out");
+  TORCH_CHECK(x.dim() == 2 && x.is_contiguous(), "x [T, width] f32 contiguous");
+  const int64_t T = x.size(0), H = x.size(1);
+  TORCH_CHECK(w.numel() == H && b.numel() == H && w.is_contiguous() && b.is_contiguous(), "norm weight / bias [width]");
+  TORCH_CHECK(out.is_contiguous() && out.dim() == 2 && out.size(0) == T && out.size(1) == H, "out [T, width]");
+  auto act2d = [&](const torch::Tensor& t, const char* what) {
+    check_rows2d(t, what);
+    TORCH_CHECK(t.is_cuda() && t.scalar_type() == out.scalar_type() && t.size(0) == T && t.size(1) == H, what,
+                ": [T, width] in the dtype of out");
+  };
+  auto vec = [&](const torch::Tensor& t, const char* what) {
+    check_f32(t, what);
+    TORCH_CHECK(t.is_contiguous() && t.numel() == H, what, ": [width] f32");
+  };
+  const void *yp = nullptr, *y2p = nullptr, *hp = nullptr;
+  const float *lsp = nullptr, *bp = nullptr, *g2p = nullptr, *hwp = nullptr;
+  long ldy = 0, ldy2 = 0, ldg2 = 0, ldh = 0;
+  TORCH_CHECK(y.has_value() || !(ls || bias || y2 || g2 || h || hw), "terms without y");
+  if (y) { act2d(*y, "y"); yp = y->data_ptr(); ldy = y->stride(0); }
+  if (ls) { vec(*ls, "ls"); lsp = ls->data_ptr<float>(); }
+  if (bias) { vec(*bias, "bias"); bp = bias->data_ptr<float>(); }
+  if (y2) { act2d(*y2, "y2"); y2p = y2->data_ptr(); ldy2 = y2->stride(0); }
+  if (g2) {
+    check_dev(*g2, "g2");
+    TORCH_CHECK(g2->scalar_type() == torch::kFloat32 && y2.has_value() && g2->dim() == 1 && g2->size(0) == T,
+                "g2 [T] f32 (may be a column of a matrix), with y2");
+    g2p = g2->data_ptr<float>();
+    ldg2 = g2->stride(0);
+  }
+  TORCH_CHECK(h.has_value() == hw.has_value(), "h and hw come together");
+  if (h) {
+    act2d(*h, "h");
+    check_f32(*hw, "hw");
+    TORCH_CHECK(hw->is_contiguous() && hw->numel() == T, "hw [T] f32");
+    hp = h->data_ptr();
+    ldh = h->stride(0);
+    hwp = hw->data_ptr<float>();
+  }
+  const int rc = dllm_ls_resadd_ln(yp, ldy, f, lsp, bp, y2p, ldy2, g2p, ldg2, hp, ldh, hwp, x.data_ptr<float>(),
+                                   w.data_ptr<float>(), b.data_ptr<float>(), out.data_ptr(), (long)T, (int)H, (float)eps,
+                                   stream());
+  ok(rc, "ls_resadd_ln");
+}
+
+void glu_act(torch::Tensor gu, c10::optional<torch::Tensor> bias, int64_t mode, double limit, double alpha, torch::Tensor y) {
+  const bool f = act_f32(gu, "gu");
+  check_rows2d(gu, "gu");
+  TORCH_CHECK(gu.size(1) % 2 == 0 && (mode == 0 || mode == 1), "gu [T, 2 ff]; mode 0 or 1");
+  const int64_t ff = gu.size(1) / 2;
+  TORCH_CHECK(y.is_cuda() && y.scalar_type() == gu.scalar_type() && y.is_contiguous() && y.dim() == 2 &&
+                  y.size(0) == gu.size(0) && y.size(1) == ff,
+              "y [T, ff]");
+  const float* bp = nullptr;
+  if (bias) {
+    check_f32(*bias, "bias");
+    TORCH_CHECK(bias->is_contiguous() && bias->numel() == 2 * ff, "bias [2 ff]");
+    bp = bias->data_ptr<float>();
+  }
+  ok(dllm_glu_act(gu.data_ptr(), gu.stride(0), f, bp, (int)ff, (int)mode, (float)limit, (float)alpha, y.data_ptr(),
+                  (long)gu.size(0), stream()),
+     "glu_act");
+}
+
+void proj_norm_prep(torch::Tensor proj, int64_t H, int64_t G, int64_t d, int64_t dv, torch::Tensor qw, torch::Tensor kw,
+                    torch::Tensor cos_sin, int64_t rot, bool interleaved, double eps, torch::Tensor qscale, bool vnorm,
+                    torch::Tensor pos, torch::Tensor slots, c10::optional<torch::Tensor> kc, c10::optional<torch::Tensor> vc,
+                    torch::Tensor q) {
+  const bool f = act_f32(proj, "proj");
+  check_rows2d(proj, "proj");
+  check_f32(cos_sin, "cos_sin");
+  check_f32(qw, "q norm weight");
+  check_f32(kw, "k norm weight");
+  check_f32(qscale, "q scale");
+  check_i32(pos, "positions");
+  check_i32(slots, "slots");
+  const int64_t T = proj.size(0);
+  const bool own = kc.has_value();
+  TORCH_CHECK(own == vc.has_value(), "both caches or none");
+  const int64_t cols = H * d + (own ? G * (d + dv) : 0);
+  TORCH_CHECK(H >= 1 && G >= 1 && H % G == 0 && d >= 1 && dv >= 1 && proj.size(1) >= cols, "proj [T, q | k | v]");
+  TORCH_CHECK(cos_sin.dim() == 2 && cos_sin.is_contiguous() && rot >= 0 && rot % 2 == 0 && rot <= d &&
+                  (rot == 0 || cos_sin.size(1) >= rot),
+              "rotation table");
+  TORCH_CHECK(qw.is_contiguous() && qw.numel() == H * d && (!own || (kw.is_contiguous() && kw.numel() == G * d)) &&
+                  qscale.is_contiguous() && qscale.numel() == H && pos.numel() == T && slots.numel() == T,
+              "norm weights [H d] / [G d], q scale [H], positions / slots [T]");
+  void *kp = nullptr, *vp = nullptr;
+  int bsz = 16;
+  if (own) {
+    for (auto* c : {&*kc, &*vc})
+      TORCH_CHECK(c->is_cuda() && c->scalar_type() == proj.scalar_type() && c->is_contiguous() && c->dim() == 4,
+                  "paged caches K [blocks, G, block, d], V [blocks, G, dv, block] in the activations' dtype");
+    TORCH_CHECK(kc->size(1) == G && vc->size(1) == G && kc->size(3) == d && vc->size(2) == dv && kc->size(0) == vc->size(0) &&
+                    kc->size(2) == vc->size(3),
+                "cache shapes");
+    kp = kc->data_ptr();
+    vp = vc->data_ptr();
+    bsz = (int)kc->size(2);
+  }
+  TORCH_CHECK(q.is_cuda() && q.scalar_type() == proj.scalar_type() && q.is_contiguous() && q.numel() == T * H * d, "q [T, H, d]");
+  ok(dllm_proj_norm_prep(proj.data_ptr(), proj.stride(0), f, (int)H, (int)G, (int)d, (int)dv, qw.data_ptr<float>(),
+                         kw.data_ptr<float>(), cos_sin.data_ptr<float>(), (int)cos_sin.size(1), (int)rot, (int)interleaved,
+                         (float)eps, qscale.data_ptr<float>(), (int)vnorm, pos.data_ptr<int>(), slots.data_ptr<int>(), kp, vp,
+                         q.data_ptr(), (long)T, bsz, stream()),
+     "proj_norm_prep");
+}
+
 void softcap(torch::Tensor x, double cap, torch::Tensor y) {
   const bool f = act_f32(x, "x");
   check_f32(y, "y");
@@ -1996,6 +2145,10 @@ PYBIND11_MODULE(_hip_kernels, m) {
   m.def("polynorm", &polynorm);
   m.def("group_router", &group_router);
   m.def("swiglu_scale", &swiglu_scale);
+  m.def("route_topk", &route_topk);
+  m.def("ls_resadd_ln", &ls_resadd_ln);
+  m.def("glu_act", &glu_act);
+  m.def("proj_norm_prep", &proj_norm_prep);
   m.def("softcap", &softcap);
   m.def("gated_group_norm", &gated_group_norm);
   m.def("outer_scan_cols", []() { return dllm_outer_scan_cols(); });
@@ -2004,7 +2157,7 @@ PYBIND11_MODULE(_hip_kernels, m) {
   m.def("qk_norm_prep", &qk_norm_prep);
   m.def("diff_combine", &diff_combine);
   m.def("causal_conv_silu", &causal_conv_silu, py::arg("x"), py::arg("w"), py::arg("b"), py::arg("state"), py::arg("qstart"),
-        py::arg("qlen"), py::arg("ctx"), py::arg("rows"), py::arg("y"), py::arg("refill") = false);
+        py::arg("qlen"), py::arg("ctx"), py::arg("rows"), py::arg("y"), py::arg("refill") = false, py::arg("act") = 0);
   m.def("selective_scan", &selective_scan);
   m.def("retention", &retention, py::arg("qkvg"), py::arg("heads"), py::arg("dim"), py::arg("vdim"), py::arg("cos_sin"),
         py::arg("rot"), py::arg("decay"), py::arg("state"), py::arg("eps"), py::arg("positions"), py::arg("qstart"),
@@ -2023,7 +2176,7 @@ PYBIND11_MODULE(_hip_kernels, m) {
   m.def("paged_gqa_attention", &paged_gqa_attention, py::arg("q"), py::arg("k_cache"), py::arg("v_cache"),
         py::arg("block_tables"), py::arg("qstart"), py::arg("qlen"), py::arg("ctx"), py::arg("tile_seq"),
         py::arg("tile_tok0"), py::arg("gate"), py::arg("out"), py::arg("mfma"), py::arg("splits") = 1,
-        py::arg("part") = py::none(), py::arg("window") = 0);
+        py::arg("part") = py::none(), py::arg("window") = 0, py::arg("keep_first") = 0, py::arg("sink") = 0.0);
   m.def("gqa_tile_tokens",
         [](int64_t H, int64_t G, bool mfma) { return (int64_t)dllm_gqa_tile_tokens((int)H, (int)G, (int)mfma); });
   m.def("gqa_mfma_ok", [](bool f32, int64_t H, int64_t G, int64_t d, int64_t dv, int64_t bs) {

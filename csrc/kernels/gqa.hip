@@ -7,6 +7,9 @@
 //               rotation, and `maps` score maps per head (differential attention: 2): query rows of
 //               one key/value head leave ordered (map, head in group), so the grouped-query kernels
 //               below pair them with key head (kv head, map); diff_combine merges the two maps.
+//   proj_norm_prep  attention inputs whose q / k RMS norm runs over the whole projection (all heads
+//               together, weights of that length) before the rotation; rotary pairs (2i, 2i + 1) or
+//               (i, i + rot / 2); a per-head q scale; optionally every value head to unit RMS.
 //   paged_gqa   one workgroup per (tile of new tokens, key/value head, group of <= 16 query heads):
 //               its rows are tokens x query heads of the group (<= 16).  Keys are walked in tiles
 //               staged in LDS as f32; a lane owns a key for the scores (one K read feeds the wave's
@@ -20,6 +23,10 @@
 //               layout (row maxima over the 16 lanes of a DPP row); the weights go through the wave's
 //               own LDS patch as bf16 hi + lo parts, so the weighted sum sees them to 16 bits of
 //               mantissa through two MFMAs.  Key blocks above a wave's newest row are skipped.
+//
+// Both attention kernels take a window (a row at position p sees keys p - win < j <= p), kept first
+// keys (j < keep stays visible at any distance; the tiles between the kept keys and the window are
+// not read) and a sink (one more term exp(0) times `sink` in the denominator, with no value).
 //
 // Cache layout: K [blocks, G, block, d], V [blocks, G, dv, block] (bf16 or f32 like the activations;
 // V is kept transposed inside its page because the weighted sum runs over keys); every score,
@@ -144,6 +151,67 @@ __global__ void __launch_bounds__(256) qk_norm_prep_kernel(const T* __restrict__
   }
 }
 
+// One workgroup per token.  q (H d entries) and k (G d entries) are each normed over their whole
+// length with weights qw / kw, then rotated on the first `rot` dims of every head: pairs (2i, 2i + 1)
+// when `inter`, else (i, i + rot / 2), angle index i; q times qscale[head].  vnorm: every value head
+// divided by its root mean square.  kc null: proj holds q alone.
+template <typename T>
+__global__ void __launch_bounds__(256) proj_norm_prep_kernel(const T* __restrict__ proj, long ld, int H, int G, int d, int dv,
+                                                             const float* __restrict__ qw, const float* __restrict__ kw,
+                                                             const float* __restrict__ cos_sin, int tab_w, int rot,
+                                                             int inter, float eps, const float* __restrict__ qscale,
+                                                             int vnorm, const int* __restrict__ pos,
+                                                             const int* __restrict__ slots, T* __restrict__ kc,
+                                                             T* __restrict__ vc, T* __restrict__ q, int BSZ) {
+  __shared__ float red[16];
+  const long tok = blockIdx.x;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const T* r = proj + tok * ld;
+  const int slot = kc ? slots[tok] : -1;
+  const long blk = slot >= 0 ? slot / BSZ : 0;
+  const int off = slot >= 0 ? slot % BSZ : 0;
+  const int half = rot >> 1;
+  const float* cs = cos_sin + (long)pos[tok] * tab_w;
+  const int nq = H * d, nk = slot >= 0 ? G * d : 0;
+  float sq = 0.f, sk = 0.f;
+  for (int e = tid; e < nq; e += 256) { const float v = ldf(r + e); sq += v * v; }
+  for (int e = tid; e < nk; e += 256) { const float v = ldf(r + nq + e); sk += v * v; }
+  const float rq = 1.f / sqrtf(block_sum(sq, red) / (float)nq + eps);
+  const float rk = nk ? 1.f / sqrtf(block_sum(sk, red) / (float)nk + eps) : 0.f;   // slot is uniform in the workgroup
+  for (int e = tid; e < nq + nk; e += 256) {
+    const bool is_q = e < nq;
+    const int c = is_q ? e : e - nq;           // column inside q or k
+    const int hh = c / d, i = c % d;
+    const T* x = r + (is_q ? 0 : nq);
+    const float* w = is_q ? qw : kw;
+    const float sc = is_q ? rq : rk;
+    float v = ldf(x + c) * sc * w[c];
+    if (i < rot) {
+      int j, f;
+      bool first;
+      if (inter) { j = i ^ 1; f = i >> 1; first = !(i & 1); }
+      else { first = i < half; j = first ? i + half : i - half; f = first ? i : i - half; }
+      const float cc = cs[f], sn = cs[half + f];
+      const float pv = ldf(x + c - i + j) * sc * w[c - i + j];
+      v = first ? v * cc - pv * sn : v * cc + pv * sn;
+    }
+    if (is_q) stf(q + (tok * H + hh) * d + i, v * qscale[hh]);
+    else stf(kc + ((blk * G + hh) * BSZ + off) * d + i, v);
+  }
+  if (slot >= 0) {   // values: a wave per value head
+    const T* vv = r + nq + nk;
+    for (int g = wave; g < G; g += 4) {
+      float sv = 1.f;
+      if (vnorm) {
+        float ss = 0.f;
+        for (int i = lane; i < dv; i += 64) { const float v = ldf(vv + g * dv + i); ss += v * v; }
+        sv = 1.f / sqrtf(wave_sum(ss) / (float)dv + eps);
+      }
+      for (int i = lane; i < dv; i += 64) stf(vc + ((blk * G + g) * dv + i) * BSZ + off, ldf(vv + g * dv + i) * sv);
+    }
+  }
+}
+
 // a [T, G, 2, R, dv] f32 (the two maps' outputs) -> out [T, G R, dv] = unit-RMS(a1 - lam a2) * scale:
 // one wave per (token, head)
 template <typename T>
@@ -176,9 +244,10 @@ __global__ void __launch_bounds__(256) paged_gqa_kernel(const T* __restrict__ q,
                                                         const int* __restrict__ tile_seq, const int* __restrict__ tile_tok0,
                                                         const T* __restrict__ gate, long ldg, T* __restrict__ out, int H,
                                                         int G, int d, int dv, int TQ, int KT, int win, int GV,
-                                                        float* __restrict__ out32) {
-  // win > 0: a row at position p sees keys p - win < j <= p.  GV value heads: key head g reads value
-  // head g / (G / GV).  out32: the output stays f32.
+                                                        float* __restrict__ out32, int keep, float sink) {
+  // win > 0: a row at position p sees keys p - win < j <= p, and keys j < keep.  GV value heads: key
+  // head g reads value head g / (G / GV).  out32: the output stays f32.  sink: one more term of score 0
+  // and that weight in the denominator.
   extern __shared__ float sm[];
   const int s = tile_seq[blockIdx.x];
   const int n = qlen[s];
@@ -216,7 +285,8 @@ __global__ void __launch_bounds__(256) paged_gqa_kernel(const T* __restrict__ q,
   const int* btr = bt + (long)s * bt_ld;
   const int gv = g / (G / GV);
   const int first = win > 0 ? max(0, p0 + tok0 - win + 1) : 0;   // the oldest key any row sees
-  for (int k0 = first / KT * KT; k0 <= last; k0 += KT) {
+  for (int k0 = (keep > 0 ? 0 : first / KT * KT); k0 <= last; k0 += KT) {
+    if (k0 >= keep && k0 + KT <= first) continue;   // between the kept keys and the window (uniform in the workgroup)
     const int nk = min(KT, last + 1 - k0);
     __syncthreads();   // the previous tile is consumed (and Qs is written)
     for (int e = tid; e < KT * d; e += 256) {
@@ -252,7 +322,7 @@ __global__ void __launch_bounds__(256) paged_gqa_kernel(const T* __restrict__ q,
     const int pk = k0 + lane;
 #pragma unroll
     for (int x = 0; x < 4; ++x) {
-      const bool vis = lane < nk && pk <= rpos[x] && (win <= 0 || pk > rpos[x] - win);
+      const bool vis = lane < nk && pk <= rpos[x] && (win <= 0 || pk > rpos[x] - win || pk < keep);
       const float sv = vis ? sc[x] : -INFINITY;
       const float mn = fmaxf(m[x], wave_max(sv));
       float p = 0.f, f = 1.f;
@@ -286,7 +356,7 @@ __global__ void __launch_bounds__(256) paged_gqa_kernel(const T* __restrict__ q,
     if (rr >= nrows) continue;
     const long tok = q0 + tok0 + rr / Rh;
     const int h = g * R + r0 + rr % Rh;
-    const float inv = 1.f / l[x];
+    const float inv = 1.f / (l[x] + (sink > 0.f ? sink * expf(-m[x]) : 0.f));
 #pragma unroll
     for (int jj = 0; jj < NJ; ++jj) {
       const int jx = lane + 64 * jj;
@@ -333,7 +403,7 @@ __global__ void __launch_bounds__(256) paged_gqa_mfma_kernel(const u16* __restri
                                                              const int* __restrict__ tile_tok0, const u16* __restrict__ gate,
                                                              long ldg, u16* __restrict__ out, int H, int G, int d, int dv,
                                                              int TQ, int splits, float* __restrict__ part, int win, int GV,
-                                                             float* __restrict__ out32) {
+                                                             float* __restrict__ out32, int keep, float sink) {
   constexpr int DS = SZ / 32, VB = SZ / 16, NKB = GM_KT / 16;
   constexpr int KSTR = SZ + 8, VSTR = GM_KT + 8, PSTR = GM_KT + 8;
   extern __shared__ __attribute__((aligned(16))) unsigned char smraw[];
@@ -421,12 +491,17 @@ __global__ void __launch_bounds__(256) paged_gqa_mfma_kernel(const u16* __restri
   };
   // small grids (decode steps) split a row's key tiles over `splits` workgroups; each leaves its
   // running maximum, sum and unnormalised output in `part`, gqa_combine merges them
-  const int tfirst = win > 0 ? max(0, p0 + tok0 - win + 1) / GM_KT : 0;   // the oldest tile any row sees
-  const int ntiles = last / GM_KT + 1 - tfirst;
-  const int kbeg = (tfirst + (int)((long)ntiles * blockIdx.z / splits)) * GM_KT;
-  const int kend = (tfirst + (int)((long)ntiles * (blockIdx.z + 1) / splits)) * GM_KT;   // exclusive
-  if (kbeg < kend) fetch(kbeg);
-  for (int k0 = kbeg; k0 < kend; k0 += GM_KT) {
+  const int tfirst = win > 0 ? max(0, p0 + tok0 - win + 1) / GM_KT : 0;   // the oldest tile of the window any row sees
+  // kept first keys: their tiles come before the window's in the walk; tile number v of the walk is
+  // tile v of the sequence for v < nkeep, else tile tfirst + v - nkeep
+  const int nkeep = win > 0 ? min(tfirst, (keep + GM_KT - 1) / GM_KT) : 0;
+  const int ntiles = last / GM_KT + 1 - tfirst + nkeep;
+  const int vbeg = (int)((long)ntiles * blockIdx.z / splits);
+  const int vend = (int)((long)ntiles * (blockIdx.z + 1) / splits);   // exclusive
+  auto tile_k0 = [&](int v) { return (v < nkeep ? v : tfirst + v - nkeep) * GM_KT; };
+  if (vbeg < vend) fetch(tile_k0(vbeg));
+  for (int vt = vbeg; vt < vend; ++vt) {
+    const int k0 = tile_k0(vt);
     __syncthreads();   // the previous tile is consumed
 #pragma unroll
     for (int f = 0; f < NF; ++f) {
@@ -436,10 +511,10 @@ __global__ void __launch_bounds__(256) paged_gqa_mfma_kernel(const u16* __restri
       const int j = e / (GM_KT / 8), cc = e % (GM_KT / 8);
       *reinterpret_cast<uint4*>(vtr + j * VSTR + 8 * cc) = pv_[f];
     }
-    if (k0 + GM_KT < kend) fetch(k0 + GM_KT);   // the next tile's loads fly under this tile's products
+    if (vt + 1 < vend) fetch(tile_k0(vt + 1));   // the next tile's loads fly under this tile's products
     __syncthreads();
     if (k0 > wave_last) continue;   // this wave's rows see nothing of the tile (the barriers above are uniform)
-    if (win > 0 && k0 + GM_KT - 1 <= wave_old - win) continue;   // ... or the tile lies before every row's window
+    if (win > 0 && k0 >= keep && k0 + GM_KT - 1 <= wave_old - win) continue;   // ... or the tile lies before every row's window
     f32x4 sacc[NKB];
 #pragma unroll
     for (int kb = 0; kb < NKB; ++kb) {
@@ -462,7 +537,8 @@ __global__ void __launch_bounds__(256) paged_gqa_mfma_kernel(const u16* __restri
       float sv[NKB];
 #pragma unroll
       for (int kb = 0; kb < NKB; ++kb)
-        sv[kb] = (full || (key0 + kb <= rpos[i] && (win <= 0 || key0 + kb > rpos[i] - win))) ? sacc[kb][i] : -INFINITY;
+        sv[kb] = (full || (key0 + kb <= rpos[i] && (win <= 0 || key0 + kb > rpos[i] - win || key0 + kb < keep)))
+                     ? sacc[kb][i] : -INFINITY;
       float mx = fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3]));
       mx = row16_max(mx);
       const float mn = fmaxf(m[i], mx);
@@ -523,7 +599,7 @@ __global__ void __launch_bounds__(256) paged_gqa_mfma_kernel(const u16* __restri
     }
     const long tok = q0 + tok0 + row / R;
     const int h = g * R + row % R;
-    const float inv = 1.f / lt;
+    const float inv = 1.f / (lt + (sink > 0.f ? sink * __expf(-m[i]) : 0.f));
 #pragma unroll
     for (int cb = 0; cb < VB; ++cb) {
       const int jx = 16 * cb + lr;
@@ -542,7 +618,7 @@ __global__ void __launch_bounds__(256) gqa_combine_kernel(const float* __restric
                                                           const int* __restrict__ tile_seq,
                                                           const int* __restrict__ tile_tok0, const u16* __restrict__ gate,
                                                           long ldg, u16* __restrict__ out, int H, int G, int dv, int TQ,
-                                                          float* __restrict__ out32) {
+                                                          float* __restrict__ out32, float sink) {
   const int s = tile_seq[blockIdx.x];
   const int n = qlen[s], tok0 = tile_tok0[blockIdx.x];
   if (n <= 0 || tok0 >= n) return;
@@ -557,7 +633,7 @@ __global__ void __launch_bounds__(256) gqa_combine_kernel(const float* __restric
     const float lz = lane < splits ? pr[lane * zs + 1] : 0.f;
     const float M = wave_max(mz);
     const float wz = mz > -INFINITY ? expf(mz - M) : 0.f;
-    const float L = wave_sum(lz * wz);
+    const float L = wave_sum(lz * wz) + (sink > 0.f ? sink * expf(-M) : 0.f);
     const long tok = qstart[s] + tok0 + row / R;
     const int h = g * R + row % R;
     for (int j0 = 0; j0 < dv; j0 += 64) {     // every lane stays in the loop: the shuffles read all lanes
@@ -594,10 +670,11 @@ long gqa_lds(int d, int dv, int KT) { return 4L * (GA_ROWS * d + (long)KT * (d |
 template <typename T, int NJ>
 int launch_gqa(dim3 grid, long lds, hipStream_t st, const T* q, const T* kc, const T* vc, const int* bt, int bt_ld, int BSZ,
                const int* qstart, const int* qlen, const int* ctx, const int* tile_seq, const int* tile_tok0, const T* gate,
-               long ldg, T* out, int H, int G, int d, int dv, int TQ, int KT, int win, int GV, float* out32) {
+               long ldg, T* out, int H, int G, int d, int dv, int TQ, int KT, int win, int GV, float* out32, int keep,
+               float sink) {
   ENSURE_LDS((paged_gqa_kernel<T, NJ>), lds);
   hipLaunchKernelGGL((paged_gqa_kernel<T, NJ>), grid, dim3(256), lds, st, q, kc, vc, bt, bt_ld, BSZ, qstart, qlen, ctx, tile_seq,
-                     tile_tok0, gate, ldg, out, H, G, d, dv, TQ, KT, win, GV, out32);
+                     tile_tok0, gate, ldg, out, H, G, d, dv, TQ, KT, win, GV, out32, keep, sink);
   return (int)hipGetLastError();
 }
 
@@ -605,8 +682,8 @@ template <typename T>
 int launch_gqa_t(int nj, dim3 grid, long lds, hipStream_t st, const void* q, const void* kc, const void* vc, const int* bt,
                  int bt_ld, int BSZ, const int* qstart, const int* qlen, const int* ctx, const int* tile_seq,
                  const int* tile_tok0, const void* gate, long ldg, void* out, int H, int G, int d, int dv, int TQ, int KT,
-                 int win, int GV, float* out32) {
-#define GQA(NJ) return launch_gqa<T, NJ>(grid, lds, st, (const T*)q, (const T*)kc, (const T*)vc, bt, bt_ld, BSZ, qstart, qlen, ctx, tile_seq, tile_tok0, (const T*)gate, ldg, (T*)out, H, G, d, dv, TQ, KT, win, GV, out32)
+                 int win, int GV, float* out32, int keep, float sink) {
+#define GQA(NJ) return launch_gqa<T, NJ>(grid, lds, st, (const T*)q, (const T*)kc, (const T*)vc, bt, bt_ld, BSZ, qstart, qlen, ctx, tile_seq, tile_tok0, (const T*)gate, ldg, (T*)out, H, G, d, dv, TQ, KT, win, GV, out32, keep, sink)
   if (nj <= 1) GQA(1);
   if (nj <= 2) GQA(2);
   GQA(4);
@@ -645,9 +722,10 @@ extern "C" int dllm_gqa_tile_tokens(int H, int G, int mfma) {
 extern "C" int dllm_paged_gqa(const void* q, const void* kc, const void* vc, int f32, const int* bt, int bt_ld, int BSZ,
                               const int* qstart, const int* qlen, const int* ctx, const int* tile_seq, const int* tile_tok0,
                               int n_tiles, const void* gate, long ldg, void* out, int H, int G, int d, int dv, int mfma,
-                              int splits, float* part, int win, int GV, int out_f32, hipStream_t st) {
+                              int splits, float* part, int win, int GV, int out_f32, int keep, float sink, hipStream_t st) {
   if (n_tiles <= 0) return 0;
-  if (G < 1 || H % G || dv > 256 || d < 1 || GV < 1 || G % GV || win < 0) return -1;
+  if (G < 1 || H % G || dv > 256 || d < 1 || GV < 1 || G % GV || win < 0 || keep < 0 || sink < 0.f) return -1;
+  if (win <= 0) keep = 0;     // without a window every key is seen anyway
   float* out32 = out_f32 ? (float*)out : nullptr;
   if (mfma) {
     if (!dllm_gqa_mfma_ok(f32, H, G, d, dv, BSZ)) return -1;
@@ -662,14 +740,14 @@ extern "C" int dllm_paged_gqa(const void* q, const void* kc, const void* vc, int
     ENSURE_LDS(paged_gqa_mfma_kernel<SZ>, lds);                                                                          \
     hipLaunchKernelGGL(paged_gqa_mfma_kernel<SZ>, grid, dim3(256), lds, st, (const u16*)q, (const u16*)kc, (const u16*)vc, bt, \
                        bt_ld, qstart, qlen, ctx, tile_seq, tile_tok0, (const u16*)gate, ldg, (u16*)out, H, G, d, dv, TQ, \
-                       splits, pp, win, GV, out32);                                                                      \
+                       splits, pp, win, GV, out32, keep, sink);                                                          \
   } while (0)
     if (sz <= 64) GQM(64); else if (sz <= 128) GQM(128); else GQM(256);
 #undef GQM
     if (pp) {
       const int rows = (TQ * (H / G) < GM_ROWS ? TQ * (H / G) : GM_ROWS);
       hipLaunchKernelGGL(gqa_combine_kernel, dim3(n_tiles, G, (rows + 3) / 4), dim3(256), 0, st, pp, splits, qstart, qlen,
-                         tile_seq, tile_tok0, (const u16*)gate, ldg, (u16*)out, H, G, dv, TQ, out32);
+                         tile_seq, tile_tok0, (const u16*)gate, ldg, (u16*)out, H, G, dv, TQ, out32, sink);
     }
     return (int)hipGetLastError();
   }
@@ -683,9 +761,9 @@ extern "C" int dllm_paged_gqa(const void* q, const void* kc, const void* vc, int
   const int TQ = dllm_gqa_tile_tokens(H, G, 0);
   if (f32)
     return launch_gqa_t<float>(nj, grid, lds, st, q, kc, vc, bt, bt_ld, BSZ, qstart, qlen, ctx, tile_seq, tile_tok0, gate, ldg,
-                               out, H, G, d, dv, TQ, KT, win, GV, out32);
+                               out, H, G, d, dv, TQ, KT, win, GV, out32, keep, sink);
   return launch_gqa_t<u16>(nj, grid, lds, st, q, kc, vc, bt, bt_ld, BSZ, qstart, qlen, ctx, tile_seq, tile_tok0, gate, ldg, out,
-                           H, G, d, dv, TQ, KT, win, GV, out32);
+                           H, G, d, dv, TQ, KT, win, GV, out32, keep, sink);
 }
 
 extern "C" int dllm_qk_norm_prep(const void* proj, long ld, int f32, const float* bias, int H, int G, int M, int d, int dv,
@@ -715,5 +793,21 @@ extern "C" int dllm_diff_combine(const float* a, void* out, int f32, long T, int
     hipLaunchKernelGGL(diff_combine_kernel<float>, grid, dim3(256), 0, st, a, (float*)out, units, H, G, dv, lam, eps, scale);
   else
     hipLaunchKernelGGL(diff_combine_kernel<u16>, grid, dim3(256), 0, st, a, (u16*)out, units, H, G, dv, lam, eps, scale);
+  return (int)hipGetLastError();
+}
+
+extern "C" int dllm_proj_norm_prep(const void* proj, long ld, int f32, int H, int G, int d, int dv, const float* qw,
+                                   const float* kw, const float* cos_sin, int tab_w, int rot, int inter, float eps,
+                                   const float* qscale, int vnorm, const int* pos, const int* slots, void* kc, void* vc, void* q,
+                                   long T, int BSZ, hipStream_t st) {
+  if (T <= 0) return 0;
+  if (rot < 0 || rot > d || (rot & 1) || rot > tab_w || H < 1 || G < 1 || H % G) return -1;
+  const dim3 grid((unsigned)T);
+  if (f32)
+    hipLaunchKernelGGL(proj_norm_prep_kernel<float>, grid, dim3(256), 0, st, (const float*)proj, ld, H, G, d, dv, qw, kw, cos_sin,
+                       tab_w, rot, inter, eps, qscale, vnorm, pos, slots, (float*)kc, (float*)vc, (float*)q, BSZ);
+  else
+    hipLaunchKernelGGL(proj_norm_prep_kernel<u16>, grid, dim3(256), 0, st, (const u16*)proj, ld, H, G, d, dv, qw, kw, cos_sin,
+                       tab_w, rot, inter, eps, qscale, vnorm, pos, slots, (u16*)kc, (u16*)vc, (u16*)q, BSZ);
   return (int)hipGetLastError();
 }

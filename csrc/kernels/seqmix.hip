@@ -22,6 +22,12 @@
 //   group_router     sigmoid scores, group-limited top-k, weights = scores: one wave per token
 //   swiglu_scale     silu(gate) * up * a per-(token, expert) weight: SwiGLU experts, dense form
 //   softcap          cap * tanh(x / cap) in f32;  gated_group_norm: rmsnorm in parts of y silu(z)
+//   ls_resadd_ln     x (f32) += ls * (y + bias + sigmoid(g) y2 + hw h), then the layer norm (mean and
+//                    variance, weight and bias) of the next sublayer's input: one workgroup per token
+//   glu_act          gated activations of a fused gate | up projection: SiLU gate, or clamped with
+//                    g sigmoid(alpha g) (u + 1)
+//   route_topk       group-limited top-k routing with sigmoid or softmax scores, a correction on the
+//                    choice and identity experts (group_router is its sigmoid / two-best form)
 //
 // Activations are bf16 or f32 (template T = u16 / float); every sum, state, norm and gate is f32.
 // Sequence metadata: qstart / qlen / ctx / rows per sequence (int32); a sequence with qlen 0 is
@@ -208,7 +214,8 @@ __global__ void __launch_bounds__(256) conv_silu_kernel(const T* __restrict__ x,
                                                         const float* __restrict__ b, const T* state,
                                                         const int* __restrict__ qstart, const int* __restrict__ qlen,
                                                         const int* __restrict__ ctx, const int* __restrict__ rows,
-                                                        T* __restrict__ y, int C, int K, T* refill) {
+                                                        T* __restrict__ y, int C, int K, T* refill, int act) {
+  // act 0: y = silu(b + conv);  act 1: y = x + b + conv (an input convolution ahead of a mixer)
   const int s = blockIdx.y;
   const int n = qlen[s];
   if (n <= 0) return;
@@ -227,7 +234,7 @@ __global__ void __launch_bounds__(256) conv_silu_kernel(const T* __restrict__ x,
       else if (p0 > 0) u = ldf(st + (long)(K - 1 + i) * C + c);
       acc += w[c * K + k] * u;
     }
-    stf(y + (long)(q0 + j) * C + c, silu_f(acc));
+    stf(y + (long)(q0 + j) * C + c, act ? acc + ldf(x + (long)(q0 + j) * ldx + c) : silu_f(acc));
   }
   // decode steps (`refill` set; every sequence brings one token, which this thread alone has read
   // the slot for): shift the slot's inputs by one and append the token's, in the same launch
@@ -702,58 +709,84 @@ __device__ __forceinline__ void wave_argmax(float& v, int& idx) {
 
 constexpr int ROUTER_MAX_E = 1024;
 
-// one wave per token: sigmoid scores, a group's score = the sum of its two best, the `top` best
-// experts inside the `keep` best groups; weights are the scores themselves
-__global__ void __launch_bounds__(256) group_router_kernel(const float* __restrict__ logits, int T, int E, int top, int count,
-                                                           int keep, int* __restrict__ ids, float* __restrict__ wts) {
-  __shared__ float sc_[4][ROUTER_MAX_E];
-  __shared__ float gs_[4][ROUTER_MAX_E];
+// One wave per token over the first E columns of its logits row.  Scores s: sigmoid (smode 0) or
+// softmax (1); choice scores c = s + corr.  `count` groups of neighbours; a group's score is the sum
+// of its two best choice scores (gmode 0) or its best (1); the `top` best c inside the `keep` best
+// groups are chosen (ties: the lower index); weights are the scores s.  Outputs >= real are identity
+// experts: their weights leave summed in idw[t], and as 0 in wts.
+__global__ void __launch_bounds__(256) route_topk_kernel(const float* __restrict__ logits, long ld, int T, int E, int top,
+                                                         int count, int keep, int smode, int gmode,
+                                                         const float* __restrict__ corr, int real, int* __restrict__ ids,
+                                                         float* __restrict__ wts, float* __restrict__ idw) {
+  __shared__ float sc_[4][ROUTER_MAX_E];     // scores
+  __shared__ float ch_[4][ROUTER_MAX_E];     // choice scores; -inf: taken
+  __shared__ float gs_[4][ROUTER_MAX_E];     // group scores; -inf: kept (taken out of the running)
+  __shared__ unsigned char ok_[4][ROUTER_MAX_E];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int t = blockIdx.x * 4 + wave;
   if (t >= T) return;
   float* sc = sc_[wave];
-  float* gs = gs_[wave];     // group score; -2: group chosen, experts allowed
-  for (int e = lane; e < E; e += 64) sc[e] = 1.f / (1.f + expf(-logits[(long)t * E + e]));
+  float* ch = ch_[wave];
+  float* gs = gs_[wave];
+  unsigned char* ok = ok_[wave];
+  const float* z = logits + (long)t * ld;
+  if (smode == 0) {
+    for (int e = lane; e < E; e += 64) sc[e] = 1.f / (1.f + expf(-z[e]));
+  } else {
+    float mx = -INFINITY;
+    for (int e = lane; e < E; e += 64) mx = fmaxf(mx, z[e]);
+    mx = wave_max(mx);
+    float sum = 0.f;
+    for (int e = lane; e < E; e += 64) { const float v = expf(z[e] - mx); sc[e] = v; sum += v; }
+    sum = wave_sum(sum);
+    for (int e = lane; e < E; e += 64) sc[e] = sc[e] / sum;
+  }
+  for (int e = lane; e < E; e += 64) ch[e] = sc[e] + (corr ? corr[e] : 0.f);
   const int per = E / count;
   const bool limited = count > 1 && keep < count;
   if (limited) {
     __builtin_amdgcn_wave_barrier();
     for (int g = lane; g < count; g += 64) {
-      float a = -1.f, b = -1.f;     // the two best (scores are in (0, 1))
+      float a = -INFINITY, b = -INFINITY;     // the two best
       for (int j = 0; j < per; ++j) {
-        const float v = sc[g * per + j];
+        const float v = ch[g * per + j];
         if (v > a) { b = a; a = v; } else if (v > b) b = v;
       }
-      gs[g] = a + (per > 1 ? b : 0.f);
+      gs[g] = (gmode == 0 && per > 1) ? a + b : a;
+      ok[g] = 0;
     }
     __builtin_amdgcn_wave_barrier();
     for (int kk = 0; kk < keep; ++kk) {
-      float bv = -1.f;
+      float bv = -INFINITY;
       int bi = 0x7fffffff;
       for (int g = lane; g < count; g += 64) {
         const float v = gs[g];
-        if (v > bv) { bv = v; bi = g; }
+        if (!ok[g] && (v > bv || bi == 0x7fffffff)) { bv = v; bi = g; }
       }
       wave_argmax(bv, bi);
-      if (lane == 0) gs[bi] = -2.f;
+      if (lane == 0) ok[bi] = 1;
       __builtin_amdgcn_wave_barrier();
     }
   }
+  float isum = 0.f;
   for (int j = 0; j < top; ++j) {
-    float bv = -1.f;
+    float bv = -INFINITY;
     int bi = 0x7fffffff;
     for (int e = lane; e < E; e += 64) {
-      const float v = sc[e];
-      if (v > bv && (!limited || gs[e / per] == -2.f)) { bv = v; bi = e; }
+      const float v = ch[e];
+      if (v > bv && (!limited || ok[e / per])) { bv = v; bi = e; }
     }
     wave_argmax(bv, bi);
     if (lane == 0) {
+      const float w = sc[bi];
       ids[(long)t * top + j] = bi;
-      wts[(long)t * top + j] = bv;
-      sc[bi] = -1.f;     // taken
+      wts[(long)t * top + j] = bi < real ? w : 0.f;
+      if (bi >= real) isum += w;
+      ch[bi] = -INFINITY;     // taken
     }
     __builtin_amdgcn_wave_barrier();
   }
+  if (lane == 0 && idw) idw[t] = isum;
 }
 
 // gu [rows, E 2 ff] (per expert: gate columns, then up columns) -> y [rows, E ff] = silu(gate) up gate[row, expert]
@@ -797,6 +830,68 @@ __global__ void __launch_bounds__(256) gated_group_norm_kernel(const float* __re
 }
 
 }  // namespace
+
+// ---------------------------------------------------------------- layer-norm layers with layer scale
+// One workgroup per token.  With y: x += ls * (y + bias + sigmoid(g2) y2 + hw h) (every term after y
+// optional; g2 and hw hold one number per token).  Then out = (x - mean) / sqrt(var + eps) * w + b with
+// the variance taken around the mean in a second pass over the row kept in LDS.
+template <typename T>
+__global__ void __launch_bounds__(256) ls_resadd_ln_kernel(const T* __restrict__ y, long ldy, const float* __restrict__ ls,
+                                                           const float* __restrict__ bias, const T* __restrict__ y2,
+                                                           long ldy2, const float* __restrict__ g2, long ldg2,
+                                                           const T* __restrict__ h, long ldh, const float* __restrict__ hw,
+                                                           float* __restrict__ x, const float* __restrict__ w,
+                                                           const float* __restrict__ b, T* __restrict__ out, int H,
+                                                           float eps) {
+  __shared__ float red[16];
+  extern __shared__ float yb[];   // [H]; entry i is touched by thread i % 256 only
+  const long row = blockIdx.x;
+  float* xr = x + row * (long)H;
+  const float s2 = (y && y2) ? (g2 ? 1.f / (1.f + expf(-g2[row * ldg2])) : 1.f) : 0.f;
+  const float sh = (y && h) ? hw[row] : 0.f;
+  float sum = 0.f;
+  for (int i = threadIdx.x; i < H; i += 256) {
+    float v = xr[i];
+    if (y) {
+      float t = ldf(y + row * ldy + i);
+      if (bias) t += bias[i];
+      if (y2) t += s2 * ldf(y2 + row * ldy2 + i);
+      if (h) t += sh * ldf(h + row * ldh + i);
+      v += ls ? ls[i] * t : t;
+      xr[i] = v;
+    }
+    yb[i] = v;
+    sum += v;
+  }
+  const float mean = block_sum(sum, red) / (float)H;
+  float sq = 0.f;
+  for (int i = threadIdx.x; i < H; i += 256) { const float dv = yb[i] - mean; sq += dv * dv; }
+  const float r = 1.f / sqrtf(block_sum(sq, red) / (float)H + eps);
+  for (int i = threadIdx.x; i < H; i += 256) stf(out + row * (long)H + i, (yb[i] - mean) * r * w[i] + b[i]);
+}
+
+// gu [rows, 2 ff] (gate columns, then up columns) + bias -> y [rows, ff].  mode 0: silu(g) u;
+// mode 1: g <- min(g, limit), u <- clamp(u, -limit, limit), y = g sigmoid(alpha g) (u + 1)
+template <typename T>
+__global__ void __launch_bounds__(256) glu_act_kernel(const T* __restrict__ gu, long ld, const float* __restrict__ bias,
+                                                      int ff, int mode, float limit, float alpha, T* __restrict__ y,
+                                                      long total) {
+  for (long e = (long)blockIdx.x * 256 + threadIdx.x; e < total; e += (long)gridDim.x * 256) {
+    const long r = e / ff;
+    const int c = (int)(e % ff);
+    float g = ldf(gu + r * ld + c), u = ldf(gu + r * ld + ff + c);
+    if (bias) { g += bias[c]; u += bias[ff + c]; }
+    float o;
+    if (mode == 0) {
+      o = silu_f(g) * u;
+    } else {
+      g = fminf(g, limit);
+      u = fminf(fmaxf(u, -limit), limit);
+      o = g / (1.f + expf(-alpha * g)) * (u + 1.f);
+    }
+    stf(y + e, o);
+  }
+}
 
 // Raise a kernel's dynamic-LDS limit when a launch needs more than it has been given so far (once per
 // size: a later launch inside a stream capture then makes no attribute call).
@@ -898,15 +993,15 @@ extern "C" int dllm_conv_refill(const void* x, long ldx, int f32, void* conv, in
 // refill != 0: a step of single tokens; the kernel also moves each token's input into its slot
 extern "C" int dllm_conv_silu(const void* x, long ldx, int f32, const float* w, const float* b, void* state,
                               const int* qstart, const int* qlen, const int* ctx, const int* rows, void* y, int T,
-                              int S, int C, int K, int refill, hipStream_t st) {
+                              int S, int C, int K, int refill, int act, hipStream_t st) {
   if (T <= 0 || S <= 0) return 0;
   if (K < 1 || K > 9) return -1;
   int gz = (T + 31) / 32;
   if (gz > 128) gz = 128;
   const dim3 g((C + 63) / 64, S, gz), blk(256);
   BY_T(f32,
-       hipLaunchKernelGGL(conv_silu_kernel<u16>, g, blk, 0, st, (const u16*)x, ldx, w, b, (const u16*)state, qstart, qlen, ctx, rows, (u16*)y, C, K, refill ? (u16*)state : nullptr),
-       hipLaunchKernelGGL(conv_silu_kernel<float>, g, blk, 0, st, (const float*)x, ldx, w, b, (const float*)state, qstart, qlen, ctx, rows, (float*)y, C, K, refill ? (float*)state : nullptr))
+       hipLaunchKernelGGL(conv_silu_kernel<u16>, g, blk, 0, st, (const u16*)x, ldx, w, b, (const u16*)state, qstart, qlen, ctx, rows, (u16*)y, C, K, refill ? (u16*)state : nullptr, act),
+       hipLaunchKernelGGL(conv_silu_kernel<float>, g, blk, 0, st, (const float*)x, ldx, w, b, (const float*)state, qstart, qlen, ctx, rows, (float*)y, C, K, refill ? (float*)state : nullptr, act))
   return (int)hipGetLastError();
 }
 
@@ -1039,14 +1134,20 @@ extern "C" int dllm_polynorm(const void* z, long ldz, int f32, const float* coef
   return (int)hipGetLastError();
 }
 
+extern "C" int dllm_route_topk(const float* logits, long ld, int T, int E, int top, int count, int keep, int smode, int gmode,
+                               const float* corr, int real, int* ids, float* wts, float* idw, hipStream_t st) {
+  if (T <= 0) return 0;
+  if (E < 1 || E > ROUTER_MAX_E || ld < E || count < 1 || E % count || keep < 1 || keep > count || top < 1 ||
+      top > keep * (E / count) || real < 0)
+    return -1;
+  hipLaunchKernelGGL(route_topk_kernel, dim3((T + 3) / 4), dim3(256), 0, st, logits, ld, T, E, top, count, keep, smode, gmode,
+                     corr, real, ids, wts, idw);
+  return (int)hipGetLastError();
+}
+
 extern "C" int dllm_group_router(const float* logits, int T, int E, int top, int count, int keep, int* ids, float* wts,
                                  hipStream_t st) {
-  if (T <= 0) return 0;
-  if (E < 1 || E > ROUTER_MAX_E || count < 1 || E % count || keep < 1 || keep > count || top < 1 ||
-      top > keep * (E / count))
-    return -1;
-  hipLaunchKernelGGL(group_router_kernel, dim3((T + 3) / 4), dim3(256), 0, st, logits, T, E, top, count, keep, ids, wts);
-  return (int)hipGetLastError();
+  return dllm_route_topk(logits, E, T, E, top, count, keep, 0, 0, nullptr, E, ids, wts, nullptr, st);
 }
 
 extern "C" int dllm_swiglu_scale(const void* gu, int f32, const float* gate, int E, int ff, void* y, long rows,
@@ -1078,5 +1179,36 @@ extern "C" int dllm_gated_group_norm(const float* y, const void* z, long ldz, in
   BY_T(f32,
        hipLaunchKernelGGL(gated_group_norm_kernel<u16>, g, dim3(256), 0, st, y, (const u16*)z, ldz, w, (u16*)out, rows, n / groups, groups, eps),
        hipLaunchKernelGGL(gated_group_norm_kernel<float>, g, dim3(256), 0, st, y, (const float*)z, ldz, w, (float*)out, rows, n / groups, groups, eps))
+  return (int)hipGetLastError();
+}
+
+extern "C" int dllm_ls_resadd_ln(const void* y, long ldy, int f32, const float* ls, const float* bias, const void* y2, long ldy2,
+                                 const float* g2, long ldg2, const void* h, long ldh, const float* hw, float* x,
+                                 const float* w, const float* b, void* out, long rows, int H, float eps, hipStream_t st) {
+  if (rows <= 0) return 0;
+  const long lds = 4L * H;
+  if (lds > 150 * 1024) return -1;
+  if (f32) {
+    ENSURE_LDS(ls_resadd_ln_kernel<float>, lds);
+    hipLaunchKernelGGL(ls_resadd_ln_kernel<float>, dim3((unsigned)rows), dim3(256), lds, st, (const float*)y, ldy, ls, bias,
+                       (const float*)y2, ldy2, g2, ldg2, (const float*)h, ldh, hw, x, w, b, (float*)out, H, eps);
+  } else {
+    ENSURE_LDS(ls_resadd_ln_kernel<u16>, lds);
+    hipLaunchKernelGGL(ls_resadd_ln_kernel<u16>, dim3((unsigned)rows), dim3(256), lds, st, (const u16*)y, ldy, ls, bias,
+                       (const u16*)y2, ldy2, g2, ldg2, (const u16*)h, ldh, hw, x, w, b, (u16*)out, H, eps);
+  }
+  return (int)hipGetLastError();
+}
+
+extern "C" int dllm_glu_act(const void* gu, long ld, int f32, const float* bias, int ff, int mode, float limit, float alpha,
+                            void* y, long rows, hipStream_t st) {
+  const long total = rows * ff;
+  if (total <= 0) return 0;
+  if (mode < 0 || mode > 1) return -1;
+  long nb = (total + 255) / 256;
+  if (nb > 65535 * 16) nb = 65535 * 16;
+  BY_T(f32,
+       hipLaunchKernelGGL(glu_act_kernel<u16>, dim3((unsigned)nb), dim3(256), 0, st, (const u16*)gu, ld, bias, ff, mode, limit, alpha, (u16*)y, total),
+       hipLaunchKernelGGL(glu_act_kernel<float>, dim3((unsigned)nb), dim3(256), 0, st, (const float*)gu, ld, bias, ff, mode, limit, alpha, (float*)y, total))
   return (int)hipGetLastError();
 }

@@ -110,7 +110,10 @@ class MixerSpec:
     ``diff``, ``kv_from`` = the layer whose cached keys / values it reads instead of its own),
     ``mamba2`` (scalar decay per head: heads, vdim, state, groups of heads sharing B / C, conv,
     norm_groups of the gated output norm) or ``mlstm`` (matrix memory with exponential gates:
-    heads, dim, vdim, gate_cap)."""
+    heads, dim, vdim, gate_cap) or ``sink_attention`` (grouped-query softmax attention with an RMS norm
+    over the whole q and k projections, rotary pairs (2i, 2i + 1), unit-RMS values, a learned number per
+    head on the scores, a sliding ``window`` that also sees the first ``keep_first`` tokens, and one
+    more term of score 0 and weight ``sink`` in the softmax denominator; ``kv_from`` as above)."""
     kind: str
     inner: int = 0
     state: int = 0
@@ -134,6 +137,8 @@ class MixerSpec:
     groups: int = 1
     norm_groups: int = 1
     gate_cap: float = 0.0
+    keep_first: int = 0
+    sink: float = 0.0
 
     @property
     def parts(self) -> Tuple["MixerSpec", ...]:
@@ -146,7 +151,7 @@ class MixerSpec:
     @property
     def paged(self) -> bool:
         return any(p.kind in ("latent_attention", "softmax_attention") or
-                   (p.kind == "diff_attention" and p.kv_from is None) for p in self.parts)
+                   (p.kind in ("diff_attention", "sink_attention") and p.kv_from is None) for p in self.parts)
 
 
 @dataclass(frozen=True)
@@ -157,7 +162,12 @@ class MoESpec:
     ``softmax`` (the chosen experts' weights renormalised) or ``sigmoid`` (weights = the chosen
     scores as they are); with ``group_count`` > 1 the experts form that many groups of neighbours,
     a group scores the sum of its two best experts and only the ``group_keep`` best groups' experts
-    can be chosen."""
+    can be chosen.  ``group_score`` "max": a group scores its best expert instead.  ``renorm`` False
+    with softmax scores: the chosen scores are the weights as they are.  ``correction``: a learned
+    vector is added to the scores for the choice (groups and experts), not for the weights.
+    ``identity`` > 0: the router has that many more outputs after the experts', standing for experts
+    that return their input.  ``shared_gate``: the shared expert's output is multiplied by the
+    sigmoid of one more projection of the token."""
     experts: int
     top: int
     scale: float
@@ -167,15 +177,24 @@ class MoESpec:
     score: str = "softmax"
     group_count: int = 1
     group_keep: int = 1
+    group_score: str = "top2"
+    renorm: bool = True
+    correction: bool = False
+    identity: int = 0
+    shared_gate: bool = False
 
 
 @dataclass(frozen=True)
 class DenseSpec:
     """One dense feed-forward ``W_down act(W_up x)``, ``ff`` wide; ``act``: ``gelu`` (the erf form) or
     ``polynorm`` (a N(z) + b N(z^2) + c N(z^3) + e with learned a, b, c, e and N the scaling of a
-    token's ff values to unit RMS)."""
+    token's ff values to unit RMS), or a gated one, ``W_down (g sigmoid(1.702 g) (u + 1))`` with
+    g = min(W_gate x, limit) and u = clamp(W_up x, -limit, limit) (``clamped_glu``).  ``bias``: every
+    projection has one."""
     ff: int
     act: str = "gelu"
+    limit: float = 0.0
+    bias: bool = False
 
 
 @dataclass(frozen=True)
@@ -206,6 +225,19 @@ class HybridConfig:
     norm_groups: int = 1
     # logits <- cap * tanh(logits / cap) (0: none)
     logit_softcap: float = 0.0
+    # with pre_norm: False leaves out the norm after a sublayer, x += sublayer(norm(x))
+    post_norm: bool = True
+    # "rms" (weight) or "layer" (mean and variance, weight and bias) for the model's norms
+    norm_kind: str = "rms"
+    # a sublayer's output is multiplied by a learned vector before it is added to the stream
+    layer_scale: bool = False
+    # taps of a causal convolution over time on every channel of the mixer's input, h <- h + conv(h)
+    # (0: none); the last taps - 1 inputs of every layer are part of a sequence's state
+    input_conv: int = 0
+    # the embedding output is multiplied by this number
+    embed_scale: float = 1.0
+    # the output projection is the embedding table
+    tied_head: bool = False
 
     @property
     def n_layers(self) -> int:
@@ -216,8 +248,13 @@ class HybridConfig:
         return any(isinstance(L.mlp, MoESpec) for L in self.layers)
 
     def num_params(self) -> int:
-        H, n = self.hidden, 2 * self.vocab * self.hidden + self.hidden
+        H, n = self.hidden, (1 if self.tied_head else 2) * self.vocab * self.hidden + self.hidden
+        nb = 2 if self.norm_kind == "layer" else 1
+        n += (nb - 1) * H
         for L in self.layers:
+            n += H * (self.input_conv + (nb - 1) + (1 if self.layer_scale else 0))
+            if L.mlp is not None:
+                n += H * ((nb - 1) + (1 if self.layer_scale else 0))
             m = L.mixer
             if m.kind == "mamba1":
                 n += 2 * m.inner * H + m.inner * (m.conv + 1) + (m.dt_rank + 2 * m.state) * m.inner
@@ -245,12 +282,22 @@ class HybridConfig:
                     n += (2 * inner + bc + m.heads) * H + (inner + bc) * (m.conv + 1) + 3 * m.heads + inner + H * inner
                 elif m.kind == "mlstm":
                     n += 2 * m.heads * m.dim * H + 3 * m.heads * m.vdim * H + m.heads * m.vdim + 2 * m.heads * (H + 1)
-            n += H * (2 if self.pre_norm else 1)
+                elif m.kind == "sink_attention":
+                    n += m.heads * m.dim * (H + 1) + m.heads + m.heads * m.vdim * H
+                    if m.kv_from is None:
+                        n += m.kv_heads * m.dim * (H + 1) + m.kv_heads * m.vdim * H
+            sides = 2 if self.pre_norm and self.post_norm else 1
+            n += H * sides
             if isinstance(L.mlp, MoESpec):
                 f = L.mlp
-                n += H + f.experts * (H + (3 if f.act == "swiglu" else 2) * f.ff * H) + 2 * f.shared_ff * H
+                mats = 3 if f.act == "swiglu" else 2
+                n += H + f.experts * (H + mats * f.ff * H) + mats * f.shared_ff * H
+                n += f.identity * H + (f.experts + f.identity if f.correction else 0) + (H if f.shared_gate else 0)
             elif isinstance(L.mlp, DenseSpec):
-                n += (2 if self.pre_norm else 1) * H + 2 * L.mlp.ff * H + (4 if L.mlp.act == "polynorm" else 0)
+                f = L.mlp
+                mats = 3 if f.act == "clamped_glu" else 2
+                n += sides * H + mats * f.ff * H + (4 if f.act == "polynorm" else 0)
+                n += (2 * f.ff + H if f.bias else 0)
         if self.depth_average:
             n += sum(i + 2 for i in range(len(self.layers)))
         return n
@@ -386,8 +433,63 @@ def pebodra_config(raw: dict, name: str = "pebodra") -> HybridConfig:
                         norm_groups=groups, logit_softcap=float(raw.get("logit_softcap") or 0.0))
 
 
+def dogilorn_config(raw: dict, name: str = "dogilorn") -> HybridConfig:
+    """A Dogilorn config.json: ``layers`` (type ``attention``, mixer sizes with ``mask.size`` /
+    ``mask.keep_first``, ``rot``, ``scale``, optional ``kv_from``; mlp ``dense`` with ``ff`` and
+    ``limit``, ``moe`` with ``expert.ff``, ``router`` (experts, identity, top, groups) and an optional
+    ``shared`` expert, or null), ``canon.taps``, ``embedding.scale``, ``norm.eps``, ``vocab``,
+    ``width``.  Layer norms with bias ahead of every sublayer, none after it, a learned scale on
+    every sublayer's output, the head tied to the embedding."""
+    layers = []
+    for i, L in enumerate(raw["layers"]):
+        m, kind = L["mixer"], L["type"]
+        if kind != "attention":
+            raise ValueError(f"unknown mixer type {kind!r}")
+        mask = m.get("mask") or {}
+        src = m.get("kv_from")
+        mix = MixerSpec("sink_attention", heads=int(m["heads"]), kv_heads=int(m.get("kv_heads", m["heads"])),
+                        dim=int(m["dim"]), vdim=int(m["vdim"]), scale=float(m["scale"]), rot=_rope(m.get("rot")),
+                        window=int(mask.get("size", 0)), keep_first=int(mask.get("keep_first", 0)), sink=1.0,
+                        kv_from=None if src is None else int(src))
+        if mix.heads % mix.kv_heads:
+            raise ValueError("heads must be a multiple of kv_heads")
+        if mix.rot is not None and (mix.rot.dims % 2 or mix.rot.dims > mix.dim):
+            raise ValueError("rot.dims must be even and at most dim")
+        if mix.kv_from is not None:
+            if not 0 <= mix.kv_from < i or layers[mix.kv_from].mixer.kv_from is not None:
+                raise ValueError(f"layer {i}: kv_from must name an earlier attention layer with keys of its own")
+            o = layers[mix.kv_from].mixer
+            if (o.kv_heads, o.dim, o.vdim, o.rot) != (mix.kv_heads, mix.dim, mix.vdim, mix.rot):
+                raise ValueError(f"layer {i}: the layer it takes keys and values from has other head sizes or rotation")
+        f = L.get("mlp")
+        mlp = None
+        if f:
+            if f["kind"] == "dense":
+                mlp = DenseSpec(int(f["ff"]), act="clamped_glu", limit=float(f["limit"]), bias=True)
+            elif f["kind"] == "moe":
+                r = f["router"]
+                g = r.get("groups") or {}
+                sh = f.get("shared")
+                mlp = MoESpec(int(r["experts"]), int(r["top"]), 1.0, int(f["expert"]["ff"]), int(sh["ff"]) if sh else 0,
+                              act="swiglu", score="softmax", group_count=int(g.get("count", 1)),
+                              group_keep=int(g.get("keep", g.get("count", 1))), group_score="max", renorm=False,
+                              correction=True, identity=int(r.get("identity", 0)), shared_gate=bool(sh))
+                outs = mlp.experts + mlp.identity
+                if outs % mlp.group_count or not 1 <= mlp.group_keep <= mlp.group_count \
+                        or mlp.top > mlp.group_keep * (outs // mlp.group_count):
+                    raise ValueError("router: experts / groups / top do not fit")
+            else:
+                raise ValueError(f"unknown feed-forward kind {f['kind']!r}")
+        layers.append(LayerSpec(mix, mlp))
+    return HybridConfig(name, "dogilorn", int(raw["width"]), int(raw["vocab"]), tuple(layers),
+                        rms_eps=float(raw["norm"]["eps"]), pre_norm=True, post_norm=False, norm_kind="layer",
+                        layer_scale=True, input_conv=int((raw.get("canon") or {}).get("taps", 0)),
+                        embed_scale=float((raw.get("embedding") or {}).get("scale", 1.0)), tied_head=True)
+
+
 # config.json "architecture" -> parser of that design's keys
-ARCHITECTURES = {"Filevik": filevik_config, "Sedopel": sedopel_config, "Pebodra": pebodra_config}
+ARCHITECTURES = {"Filevik": filevik_config, "Sedopel": sedopel_config, "Pebodra": pebodra_config,
+                 "Dogilorn": dogilorn_config}
 
 AnyConfig = Union[ModelConfig, HybridConfig]
 

@@ -42,10 +42,21 @@ they do not take and for f32 models), everything between them on the HIP kernels
              sigmoid gate in the kernel) -> out-proj
   experts    (sigmoid scores) f32 router logits -> group-limited top-k, weights = scores -> grouped
              SwiGLU expert GEMMs or their dense form
+  sink_attn  (input: h + a short causal convolution of h, its last inputs kept in the slot) one fused
+             q | k | v projection -> RMS norm over the whole q and k projections, rotary pairs
+             (2i, 2i + 1), unit-RMS values, k and v to their pages (a layer with ``kv_from`` projects q
+             alone) -> attention inside a sliding window that also keeps the first tokens, with one
+             more term of score 0 in the softmax denominator -> out-proj
+  clamped    one fused gate | up projection -> biases, clamps, g sigmoid(1.702 g) (u + 1) -> down-proj
+  experts    (softmax scores + a correction for the choice, identity experts) one f32 GEMM for the
+             router logits and the shared expert's gate logit -> group-limited top-k -> SwiGLU experts;
+             identity experts, the gated shared expert and the layer scale ride in the residual launch
 
 Layer forms: ``x += norm(sublayer(x))`` (Filevik) or, with ``cfg.pre_norm``, a norm on both sides,
-``x += norm_b(sublayer(norm(x)))``; with ``cfg.depth_average`` a layer hands on a learned weighted
-sum of the embedding output and all layer results so far (kept as an f32 stack for the step).
+``x += norm_b(sublayer(norm(x)))``, or without ``cfg.post_norm`` ``x += ls * sublayer(layernorm(x))``
+(layer norms with bias, a learned scale per channel); with ``cfg.depth_average`` a layer hands on a
+learned weighted sum of the embedding output and all layer results so far (kept as an f32 stack for
+the step).
 
 Per-sequence state lives in slots owned by the engine (its batch rows); paged latents use the
 engine's block tables.  No tensor parallelism.
@@ -86,7 +97,12 @@ class HybridModel:
         if dtype not in (torch.bfloat16, torch.float32):
             raise ValueError("dtype must be bfloat16 or float32")
         self.cfg, self.device, self.dtype, self.par = cfg, torch.device(device), dtype, par
-        self.has_recurrent_state = any(L.mixer.recurrent for L in cfg.layers)
+        if cfg.pre_norm and not cfg.post_norm and (cfg.norm_kind != "layer" or cfg.depth_average):
+            raise ValueError(f"{cfg.name}: layers without a norm after the sublayer use layer norms and no depth average")
+        if cfg.norm_kind == "layer" and (not cfg.pre_norm or cfg.post_norm):
+            raise ValueError(f"{cfg.name}: layer norms are built for the pre-norm layer form only")
+        # the input convolution's last inputs are per-sequence state like a recurrence's
+        self.has_recurrent_state = any(L.mixer.recurrent for L in cfg.layers) or cfg.input_conv > 1
         self.layers: List[Dict[str, torch.Tensor]] = []
         self.tap: Optional[list] = None      # debugging: residual stream after every layer
         self._rot: Dict[Tuple[int, float], torch.Tensor] = {}
@@ -109,12 +125,22 @@ class HybridModel:
             return rnd(n_out, n_in, s=1.0 / math.sqrt(n_in))
 
         t["embed"] = rnd(cfg.vocab, W, s=1.0)
-        t["head"] = lin(cfg.vocab, W)
+        if not cfg.tied_head:
+            t["head"] = lin(cfg.vocab, W)
         t["final.norm"] = torch.ones(W)
+        lnb = cfg.norm_kind == "layer"
+        if lnb:
+            t["final.norm.b"] = rnd(W, s=0.1)
         for i, L in enumerate(cfg.layers):
             p, m = f"l{i}.", L.mixer
             t[p + "norm1"] = torch.ones(W)
-            if cfg.pre_norm:
+            if lnb:
+                t[p + "norm1.b"] = rnd(W, s=0.1)
+            if cfg.layer_scale:
+                t[p + "ls1"] = torch.full((W,), 0.5)
+            if cfg.input_conv:
+                t[p + "canon1"] = rnd(W, cfg.input_conv, s=0.3)
+            if cfg.pre_norm and cfg.post_norm:
                 t[p + "norm1b"] = torch.ones(W)
             if cfg.depth_average:
                 t[p + "dwa"] = torch.cat([rnd(i + 1, s=0.05), torch.ones(1)])
@@ -164,6 +190,12 @@ class HybridModel:
                 t[p + "mix.i"], t[p + "mix.f"] = lin(m.heads, W), lin(m.heads, W)
                 t[p + "mix.i.b"] = rnd(m.heads, s=0.1)
                 t[p + "mix.f.b"] = torch.linspace(3.0, 6.0, m.heads)
+            elif m.kind == "sink_attention":
+                t[p + "mix.q"], t[p + "mix.q.norm"] = lin(m.heads * m.dim, W), torch.ones(m.heads * m.dim)
+                t[p + "mix.temp"], t[p + "mix.o"] = torch.ones(m.heads), lin(W, m.heads * m.vdim)
+                if m.kv_from is None:
+                    t[p + "mix.k"], t[p + "mix.k.norm"] = lin(m.kv_heads * m.dim, W), torch.ones(m.kv_heads * m.dim)
+                    t[p + "mix.v"] = lin(m.kv_heads * m.vdim, W)
             elif m.kind == "mamba1":
                 t[p + "mix.in"] = lin(2 * m.inner, W)
                 t[p + "mix.conv"] = rnd(m.inner, m.conv, s=1.0 / math.sqrt(m.conv))
@@ -186,22 +218,37 @@ class HybridModel:
                 t[p + "mix.uk"], t[p + "mix.uv"] = lin(m.heads * m.dim, m.kv_rank), lin(m.heads * m.vdim, m.kv_rank)
                 t[p + "mix.o"] = lin(W, m.heads * m.vdim)
             f = L.mlp
-            if isinstance(f, DenseSpec):
+            if f is not None:
                 t[p + "norm2"] = torch.ones(W)
-                if cfg.pre_norm:
+                if lnb:
+                    t[p + "norm2.b"] = rnd(W, s=0.1)
+                if cfg.layer_scale:
+                    t[p + "ls2"] = torch.full((W,), 0.5)
+            if isinstance(f, DenseSpec):
+                if cfg.pre_norm and cfg.post_norm:
                     t[p + "norm2b"] = torch.ones(W)
                 t[p + "mlp.up"], t[p + "mlp.down"] = lin(f.ff, W), lin(W, f.ff)
                 if f.act == "polynorm":
                     t[p + "mlp.act"] = torch.tensor([1.0, 0.5, 0.25, 0.0])
+                if f.act == "clamped_glu":
+                    t[p + "mlp.gate"] = lin(f.ff, W)
+                if f.bias:
+                    for n_, c in (("gate", f.ff), ("up", f.ff), ("down", W)):
+                        t[p + f"mlp.{n_}.b"] = rnd(c, s=0.1)
             elif f is not None:
-                t[p + "norm2"] = torch.ones(W)
-                t[p + "mlp.router"] = lin(f.experts, W)
+                t[p + "mlp.router"] = lin(f.experts + f.identity, W)
+                if f.correction:
+                    t[p + "mlp.correction"] = rnd(f.experts + f.identity, s=0.01)
                 for e in range(f.experts):
                     t[p + f"mlp.e{e}.up"], t[p + f"mlp.e{e}.down"] = lin(f.ff, W), lin(W, f.ff)
                     if f.act == "swiglu":
                         t[p + f"mlp.e{e}.gate"] = lin(f.ff, W)
                 if f.shared_ff:
                     t[p + "mlp.shared.up"], t[p + "mlp.shared.down"] = lin(f.shared_ff, W), lin(W, f.shared_ff)
+                    if f.act == "swiglu":
+                        t[p + "mlp.shared.gate"] = lin(f.shared_ff, W)
+                    if f.shared_gate:
+                        t[p + "mlp.shared.sg"] = lin(1, W)
         return t
 
     @staticmethod
@@ -223,14 +270,26 @@ class HybridModel:
         put = lambda x: x.to(dev, dt).contiguous()
         f32 = lambda x: x.to(dev, torch.float32).contiguous()
         W = cfg.hidden
-        self.embed, self.lm_head, self.final_norm = put(t["embed"]), put(t["head"]), f32(t["final.norm"])
+        self.embed, self.final_norm = put(t["embed"]), f32(t["final.norm"])
+        self.lm_head = self.embed if cfg.tied_head else put(t["head"])      # tied: the table itself, unscaled
+        lnb = cfg.norm_kind == "layer"
+        self.final_norm_b = f32(t["final.norm.b"]) if lnb else None
         if tuple(self.embed.shape) != (cfg.vocab, W) or tuple(self.lm_head.shape) != (cfg.vocab, W):
             raise ValueError("embed / head do not fit config vocab x width")
         for i, L in enumerate(cfg.layers):
             p, m = f"l{i}.", L.mixer
             D: Dict[str, torch.Tensor] = {"norm1": f32(t[p + "norm1"])}
-            if cfg.pre_norm:
+            if cfg.pre_norm and cfg.post_norm:
                 D["norm1b"] = f32(t[p + "norm1b"])
+            if lnb:
+                D["norm1.b"] = f32(t[p + "norm1.b"])
+            if cfg.layer_scale:
+                D["ls1"] = f32(t[p + "ls1"])
+                assert D["ls1"].numel() == W
+            if cfg.input_conv:
+                D["canon"] = f32(t[p + "canon1"])
+                D["canon_b"] = torch.zeros(W, dtype=torch.float32, device=dev)
+                assert tuple(D["canon"].shape) == (W, cfg.input_conv)
             if cfg.depth_average:
                 D["dwa"] = f32(t[p + "dwa"])
                 assert D["dwa"].numel() == i + 2
@@ -268,6 +327,17 @@ class HybridModel:
                 cols = 2 * m.heads * m.dim + ((2 * m.kv_heads * m.dim + m.kv_heads * m.vdim) if own else 0)
                 assert D["proj"].shape[0] == cols == D["bias"].numel() and D["qnorm"].numel() == m.dim
                 assert tuple(D["o"].shape) == (W, m.heads * m.vdim)
+            elif m.kind == "sink_attention":
+                own = m.kv_from is None
+                D["proj"] = put(torch.cat([t[p + "mix." + n] for n in (("q", "k", "v") if own else ("q",))], 0))
+                D["qnorm"] = f32(t[p + "mix.q.norm"])
+                D["knorm"] = f32(t[p + "mix.k.norm"]) if own else D["qnorm"]
+                D["qscale"] = f32(t[p + "mix.temp"]) * m.scale         # score scale times the head's number
+                D["o"] = put(t[p + "mix.o"])
+                cols = m.heads * m.dim + (m.kv_heads * (m.dim + m.vdim) if own else 0)
+                assert D["proj"].shape[0] == cols and D["qnorm"].numel() == m.heads * m.dim and D["qscale"].numel() == m.heads
+                assert not own or D["knorm"].numel() == m.kv_heads * m.dim
+                assert tuple(D["o"].shape) == (W, m.heads * m.vdim)
             elif m.kind == "mamba2":
                 inner, bc = m.heads * m.vdim, 2 * m.groups * m.state
                 D["in"], D["o"] = put(t[p + "mix.in"]), put(t[p + "mix.o"])
@@ -299,19 +369,40 @@ class HybridModel:
                 D["uk"] = put(t[p + "mix.uk"].view(m.heads, m.dim, m.kv_rank))                       # [H, d, r]
                 D["uvT"] = put(t[p + "mix.uv"].view(m.heads, m.vdim, m.kv_rank).transpose(1, 2))    # [H, r, dv]
             f = L.mlp
+            if f is not None:
+                if lnb:
+                    D["norm2.b"] = f32(t[p + "norm2.b"])
+                if cfg.layer_scale:
+                    D["ls2"] = f32(t[p + "ls2"])
             if isinstance(f, DenseSpec):
-                D["norm2"], D["up"], D["down"] = f32(t[p + "norm2"]), put(t[p + "mlp.up"]), put(t[p + "mlp.down"])
-                if cfg.pre_norm:
+                D["norm2"], D["down"] = f32(t[p + "norm2"]), put(t[p + "mlp.down"])
+                if f.act == "clamped_glu":     # one projection: gate rows, then up rows
+                    D["up"] = put(torch.cat([t[p + "mlp.gate"], t[p + "mlp.up"]], 0))
+                    assert tuple(D["up"].shape) == (2 * f.ff, W)
+                else:
+                    D["up"] = put(t[p + "mlp.up"])
+                    assert tuple(D["up"].shape) == (f.ff, W)
+                if f.bias:
+                    names = ("gate", "up") if f.act == "clamped_glu" else ("up",)
+                    D["up_b"] = f32(torch.cat([t[p + f"mlp.{n}.b"] for n in names], 0))
+                    D["down_b"] = f32(t[p + "mlp.down.b"])
+                    assert D["up_b"].numel() == D["up"].shape[0] and D["down_b"].numel() == W
+                if cfg.pre_norm and cfg.post_norm:
                     D["norm2b"] = f32(t[p + "norm2b"])
-                assert tuple(D["up"].shape) == (f.ff, W)
                 if f.act == "polynorm":
                     D["act"] = f32(t[p + "mlp.act"])
                     assert D["act"].numel() == 4
             elif f is not None:
                 D["norm2"] = f32(t[p + "norm2"])
                 D["router"] = put(t[p + "mlp.router"])
-                if f.score == "sigmoid":
+                if f.score == "sigmoid" or not f.renorm:
                     D["router"] = f32(t[p + "mlp.router"])     # the router runs in f32
+                    assert tuple(D["router"].shape) == (f.experts + f.identity, W)
+                if f.shared_gate:     # the shared expert's gate logit is one more row of the router's GEMM
+                    D["router"] = torch.cat([D["router"], f32(t[p + "mlp.shared.sg"]).view(1, W)], 0).contiguous()
+                if f.correction:
+                    D["corr"] = f32(t[p + "mlp.correction"])
+                    assert D["corr"].numel() == f.experts + f.identity
                 if f.act == "swiglu":      # per expert: gate rows, then up rows
                     w1 = torch.stack([torch.cat([t[p + f"mlp.e{e}.gate"], t[p + f"mlp.e{e}.up"]], 0)
                                       for e in range(f.experts)])                         # [E, 2 ff, W]
@@ -332,10 +423,14 @@ class HybridModel:
                     D["w2d"] = put(w2.permute(1, 0, 2).reshape(W, f.experts * f.ff))
                 if f.shared_ff:
                     D["sh_up"], D["sh_down"] = put(t[p + "mlp.shared.up"]), put(t[p + "mlp.shared.down"])
+                    if f.act == "swiglu":     # gate rows, then up rows
+                        D["sh_up"] = put(torch.cat([t[p + "mlp.shared.gate"], t[p + "mlp.shared.up"]], 0))
+                    assert D["sh_down"].shape[1] == f.shared_ff
             self.layers.append(D)
 
     def weight_bytes(self) -> int:
-        n = sum(x.numel() * x.element_size() for x in (self.embed, self.lm_head, self.final_norm))
+        n = sum(x.numel() * x.element_size() for x in (self.embed, self.final_norm))
+        n += 0 if self.cfg.tied_head else self.lm_head.numel() * self.lm_head.element_size()
         return n + sum(x.numel() * x.element_size() for L in self.layers for x in L.values() if torch.is_tensor(x))
 
     def decode_read_bytes(self, top_only: bool = True) -> int:
@@ -378,6 +473,8 @@ class HybridModel:
                     n += block_size * m.kv_heads * (m.dim + m.vdim) * it
                 elif m.kind == "diff_attention" and m.kv_from is None:
                     n += block_size * m.kv_heads * (2 * m.dim + m.vdim) * it
+                elif m.kind == "sink_attention" and m.kv_from is None:
+                    n += block_size * m.kv_heads * (m.dim + m.vdim) * it
         return n
 
     def alloc_caches(self, num_blocks: int, block_size: int, slots: int) -> List[tuple]:
@@ -390,11 +487,20 @@ class HybridModel:
         values [blocks, kv_heads, vdim, block]), for a layer with ``kv_from`` the tensors of that
         layer / mamba2: (conv inputs [slots, taps - 1, x | B | C channels], state [slots, heads, N,
         vdim] f32) / mlstm: (memory [slots, heads, dim, vdim] f32, normaliser and maximum [slots,
-        heads, column blocks, dim + 1] f32)."""
+        heads, column blocks, dim + 1] f32) / sink_attention: (paged keys [blocks, kv_heads, block,
+        dim], paged values [blocks, kv_heads, vdim, block]), of the layer ``kv_from`` names if any.
+        With an input convolution every layer's tuple ends with its own last inputs [slots, taps - 1,
+        width]."""
         dev, out = self.device, []
         for L in self.cfg.layers:
             m = L.mixer
-            if m.kind == "diff_attention":
+            if m.kind == "sink_attention":
+                if m.kv_from is not None:
+                    out.append(out[m.kv_from][:2])
+                else:
+                    out.append((torch.zeros((num_blocks, m.kv_heads, block_size, m.dim), dtype=self.dtype, device=dev),
+                                torch.zeros((num_blocks, m.kv_heads, m.vdim, block_size), dtype=self.dtype, device=dev)))
+            elif m.kind == "diff_attention":
                 if m.kv_from is not None:
                     out.append(out[m.kv_from])
                 else:
@@ -424,6 +530,9 @@ class HybridModel:
                 out.append((torch.zeros((slots, m.heads, m.dim, m.vdim), dtype=torch.float32, device=dev),))
             else:
                 out.append((torch.zeros((num_blocks, block_size, m.kv_rank + m.rot_dim), dtype=self.dtype, device=dev),))
+            if self.cfg.input_conv:
+                out[-1] = out[-1] + (torch.zeros((slots, max(self.cfg.input_conv - 1, 0), self.cfg.hidden),
+                                                 dtype=self.dtype, device=dev),)
         return out
 
     # ------------------------------------------------------------------ mixers
@@ -528,6 +637,32 @@ class HybridModel:
         o = seqmix.diff_combine(a, m.heads, m.kv_heads, m.vdim, L["lam"], self.cfg.rms_eps, 1.0 - m.diff, self.dtype)
         return _mm(o, L["o"])
 
+    def _input_conv(self, L, h, meta, state):
+        """h + a short causal convolution of h over time (per channel, no activation); the slot keeps
+        the sequence's last inputs."""
+        single = meta.host_qlen is None      # a decode step: the convolution refills its slots itself
+        y = seqmix.causal_conv_silu(h, L["canon"], L["canon_b"], state, meta.qstart, meta.qlen, meta.ctx,
+                                    meta.state_rows, refill=single, act="residual")
+        if not single:
+            seqmix.conv_state_refill(h, state, meta.qstart, meta.qlen, meta.ctx, meta.state_rows)
+        return y
+
+    def _sink_attention(self, L, m: MixerSpec, x, positions, meta, cache):
+        k_cache, v_cache = cache[0], cache[1]
+        own = m.kv_from is None
+        proj = _mm(x, L["proj"])                                        # q | k | v, or q alone
+        rot = m.rot.dims if m.rot is not None else 0
+        table = self._table(m) if rot else self._any_table()
+        q = seqmix.proj_norm_prep(proj, m.heads, m.kv_heads, m.dim, m.vdim, L["qnorm"], L["knorm"], table, rot, True,
+                                  self.cfg.rms_eps, L["qscale"], True, positions, meta.slots, k_cache if own else None,
+                                  v_cache if own else None)
+        mfma = seqmix.gqa_use_mfma(q, m.heads, m.kv_heads, m.dim, m.vdim, k_cache.shape[2])
+        ts, tt = meta.latent_tiles(1, self.device, seqmix.gqa_tokens_per_tile(m.heads, m.kv_heads, mfma))
+        splits = seqmix.gqa_splits(int(ts.numel()), m.kv_heads, meta.max_ctx, m.window, m.keep_first) if mfma else 1
+        o = seqmix.paged_gqa_attention(q, k_cache, v_cache, meta.block_tables, meta.qstart, meta.qlen, meta.ctx, ts, tt,
+                                       None, mfma, splits, window=m.window, keep_first=m.keep_first, sink=m.sink)
+        return _mm(o, L["o"])
+
     def _mamba2(self, L, m: MixerSpec, x, meta, cache):
         conv_state, state = cache
         rows = meta.state_rows
@@ -552,7 +687,10 @@ class HybridModel:
 
     def _dense(self, L, f: DenseSpec, x):
         z = _mm(x, L["up"])
-        a = seqmix.polynorm(z, L["act"], self.cfg.rms_eps) if f.act == "polynorm" else seqmix.gelu_erf(z)
+        if f.act == "clamped_glu":      # the down projection's bias rides in the residual launch
+            a = seqmix.glu_act(z, L.get("up_b"), "clamped", f.limit, 1.702)
+        else:
+            a = seqmix.polynorm(z, L["act"], self.cfg.rms_eps) if f.act == "polynorm" else seqmix.gelu_erf(z)
         return _mm(a, L["down"])
 
     def _experts_swiglu(self, L, f: MoESpec, x):
@@ -563,6 +701,29 @@ class HybridModel:
         ids, w = seqmix.group_router(logits, f.top, f.group_count, f.group_keep)
         if f.scale != 1.0:
             w = w * f.scale
+        return self._swiglu_experts(L, f, x, ids, w)
+
+    def _experts_terms(self, L, f: MoESpec, x) -> dict:
+        """Softmax router in f32 whose choice (not its weights) sees a learned correction, group-limited
+        top-k over experts and identity experts together, weights = the chosen scores; returns the
+        terms of the residual launch (ops.seqmix.ls_resadd_ln): the routed experts' sum, the input
+        times the identity experts' weights, the shared expert and its gate logit."""
+        logits = F.linear(x.float(), L["router"])      # [T, experts + identity (+ 1: the shared expert's gate)]
+        R = f.experts + f.identity
+        ids, w, idw = seqmix.route_topk(logits, R, f.top, f.group_count, f.group_keep, f.score, f.group_score,
+                                        L.get("corr"), f.experts)
+        if f.scale != 1.0:
+            w, idw = w * f.scale, idw * f.scale
+        out = dict(y=self._swiglu_experts(L, f, x, ids, w))
+        if f.identity:
+            out.update(h=x, hw=idw)
+        if f.shared_ff:
+            out.update(y2=_mm(seqmix.glu_act(_mm(x, L["sh_up"])), L["sh_down"]), g2=logits[:, R] if f.shared_gate else None)
+        return out
+
+    def _swiglu_experts(self, L, f: MoESpec, x, ids, w):
+        """sum_j w[t, j] expert_(ids[t, j])(x_t); ids beyond the experts (identity experts, whose weight
+        here is 0) add nothing."""
         if L.get("tg"):
             return ops.moe_ffn_tg(x if x.stride(1) == 1 else x.contiguous(), ids, w, L["w1"], L["w2"])
         if "w2" in L and (not x.is_cuda or seqmix.moe_ffn_relu2_ok(x, L["w1"])):
@@ -613,6 +774,9 @@ class HybridModel:
         else:
             x = self.embed.index_select(0, input_ids.long())
             xl = None
+        if cfg.embed_scale != 1.0:
+            x = x * cfg.embed_scale      # f32; the pre-norm layers read their own normed copy
+            xl = None if xl is None else x.to(self.dtype)
         T, W, nL = x.shape[0], cfg.hidden, len(self.layers)
         X = None
         if cfg.depth_average:
@@ -623,12 +787,17 @@ class HybridModel:
             X[1].copy_(x)
             x = X[1]
         h = None
-        if cfg.pre_norm:
+        ln = cfg.norm_kind == "layer"
+        if ln:
+            h = seqmix.ls_resadd_ln(x, self.layers[0]["norm1"], self.layers[0]["norm1.b"], eps, self.dtype)
+        elif cfg.pre_norm:
             h = seqmix.rms_rows(x, self.layers[0]["norm1"], eps, out_dtype=self.dtype)
         for i, (L, S, cache) in enumerate(zip(self.layers, cfg.layers, kv_caches)):
             m = S.mixer
             if not cfg.pre_norm:
                 h = x if xl is None else xl
+            if cfg.input_conv:
+                h = self._input_conv(L, h, meta, cache[-1])
             if m.kind == "mamba1":
                 y = self._mamba(L, m, h, meta, cache)
             elif m.kind == "retention":
@@ -643,9 +812,22 @@ class HybridModel:
                 y = self._mamba2(L, m, h, meta, cache)
             elif m.kind == "mlstm":
                 y = self._mlstm(L, m, h, meta, cache)
+            elif m.kind == "sink_attention":
+                y = self._sink_attention(L, m, h, positions, meta, cache)
             else:
                 y = self._latent(L, m, h, positions, meta, cache)
-            if cfg.pre_norm:
+            if ln:
+                # x += ls * sublayer, and the layer norm ahead of the next sublayer, in one launch
+                nw, nb = (self.layers[i + 1]["norm1"], self.layers[i + 1]["norm1.b"]) if i + 1 < nL else \
+                    (self.final_norm, self.final_norm_b)
+                if S.mlp is not None:
+                    h = seqmix.ls_resadd_ln(x, L["norm2"], L["norm2.b"], eps, self.dtype, y=y, ls=L.get("ls1"))
+                    terms = dict(y=self._dense(L, S.mlp, h), bias=L.get("down_b")) if isinstance(S.mlp, DenseSpec) else \
+                        self._experts_terms(L, S.mlp, h)
+                    h = seqmix.ls_resadd_ln(x, nw, nb, eps, self.dtype, ls=L.get("ls2"), **terms)
+                else:
+                    h = seqmix.ls_resadd_ln(x, nw, nb, eps, self.dtype, y=y, ls=L.get("ls1"))
+            elif cfg.pre_norm:
                 # the sublayer's tail and the next sublayer's input norm in one launch
                 nxt = self.layers[i + 1]["norm1"] if i + 1 < nL else self.final_norm
                 pair = dict(b=y[1], wa=L["lout"], wb=L["rout"]) if isinstance(y, tuple) else {}

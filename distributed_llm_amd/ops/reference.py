@@ -175,9 +175,11 @@ def moe_gate(logits, k):
 
 def moe_ffn(x, ids, wts, w13, w2):
     """sum_j wts[t, j] * (silu(x w13_e[:I]^T) * (x w13_e[I:]^T)) w2_e^T  with e = ids[t, j] (f32 math,
-    bf16 rounding of the activation like the kernel)."""
+    bf16 rounding of the activation like the kernel).  Ids outside [0, E) are clamped like the
+    kernel's routing does (callers give such pairs the weight 0)."""
     T, H = x.shape
     I = w13.shape[1] // 2
+    ids = ids.clamp(0, w13.shape[0] - 1)
     out = torch.zeros((T, H), dtype=torch.float32, device=x.device)
     xf = x.float()
     for j in range(ids.shape[1]):
@@ -394,10 +396,11 @@ def norm_resadd(y, w, eps, x, x_lp=None, groups=1, bias=None):
     return x
 
 
-def causal_conv_silu(x, w, b, conv_state, qstart, qlen, ctx, rows):
+def causal_conv_silu(x, w, b, conv_state, qstart, qlen, ctx, rows, act="silu"):
     """y[t, c] = silu(b[c] + sum_k w[c, k] u[t - K + 1 + k, c]) over each sequence's inputs u (the
     slot's last K - 1 inputs before its new tokens, zeros before position 0).  x [T, >= C] (first C
-    columns), conv_state [slots, K - 1, C].  The state is NOT updated (selective_scan does)."""
+    columns), conv_state [slots, K - 1, C].  The state is NOT updated (selective_scan does).
+    ``act`` "residual": no activation, y = x + (b + the convolution)."""
     C, K = w.shape
     y = torch.zeros((x.shape[0], C), dtype=x.dtype, device=x.device)
     wf = w.float()
@@ -407,7 +410,7 @@ def causal_conv_silu(x, w, b, conv_state, qstart, qlen, ctx, rows):
         acc = b.float()[None, :].expand(n, C).clone()
         for k in range(K):
             acc += u[k:k + n] * wf[:, k][None, :]
-        y[q0:q0 + n] = torch.nn.functional.silu(acc).to(x.dtype)
+        y[q0:q0 + n] = (torch.nn.functional.silu(acc) if act == "silu" else acc + x[q0:q0 + n, :C].float()).to(x.dtype)
     return y
 
 
@@ -611,12 +614,15 @@ def attn_prep(proj, heads, kv_heads, dim, vdim, cos_sin, rot_dims, eps, qscale, 
     return q.to(proj.dtype)
 
 
-def paged_gqa_attention(q, k_cache, v_cache, block_tables, qstart, qlen, ctx, gate=None, window=0, out_f32=False):
+def paged_gqa_attention(q, k_cache, v_cache, block_tables, qstart, qlen, ctx, gate=None, window=0, out_f32=False,
+                        keep_first=0, sink=0.0):
     """Causal softmax attention of q [T, heads, dim] (already scaled) over paged keys / values;
     query head h reads key head h // (heads / kv_heads); the output [T, heads * vdim] is
     multiplied by sigmoid(gate) when a gate [T, heads * vdim] is given.  ``window`` > 0: position i
-    sees keys i - window < j <= i.  A value cache with fewer heads than the key cache is shared by
-    neighbouring key heads (key head g reads value head g // (key heads / value heads))."""
+    sees keys i - window < j <= i, and the keys j < ``keep_first`` whatever their distance.  A value
+    cache with fewer heads than the key cache is shared by neighbouring key heads (key head g reads
+    value head g // (key heads / value heads)).  ``sink``: weight of one more term of score 0 in
+    every softmax denominator (it has no value): p_j = exp(s_j) / (sink + sum exp(s_j))."""
     T, H, d = q.shape
     G, BSz, dv = k_cache.shape[1], k_cache.shape[2], v_cache.shape[2]
     vrep = G // v_cache.shape[1]
@@ -636,9 +642,16 @@ def paged_gqa_attention(q, k_cache, v_cache, block_tables, qstart, qlen, ctx, ga
         pos = torch.arange(c - n, c, device=q.device)
         mask = torch.arange(c, device=q.device)[None, :] > pos[:, None]
         if window > 0:
-            mask = mask | (torch.arange(c, device=q.device)[None, :] <= pos[:, None] - window)
+            keys = torch.arange(c, device=q.device)[None, :]
+            mask = mask | ((keys <= pos[:, None] - window) & (keys >= keep_first))
         sc = sc.masked_fill(mask[None], float("-inf"))
-        o = torch.einsum("htu,uhv->thv", torch.softmax(sc, -1), V).reshape(n, H * dv)
+        if sink > 0:
+            mx = sc.max(-1, keepdim=True).values.clamp_min(0.0)
+            e = torch.exp(sc - mx)
+            pr = e / (e.sum(-1, keepdim=True) + sink * torch.exp(-mx))
+        else:
+            pr = torch.softmax(sc, -1)
+        o = torch.einsum("htu,uhv->thv", pr, V).reshape(n, H * dv)
         if gate is not None:
             o = o * torch.sigmoid(gate[qs[s]:qs[s] + n].float())
         out[qs[s]:qs[s] + n] = o.to(out.dtype)
@@ -851,23 +864,43 @@ def polynorm(z, coef, eps):
     return (a * N(zf) + b * N(zf * zf) + c * N(zf * zf * zf) + e).to(z.dtype)
 
 
-def group_router(logits, top, count, keep):
-    """Scores = sigmoid(logits) [T, E] f32.  The experts form ``count`` groups of neighbours; a group
-    scores the sum of its two best experts; the ``top`` best experts inside the ``keep`` best groups
-    are chosen (ties: the lower index), weights = their scores.  -> ids [T, top] int32, w [T, top] f32."""
-    s = torch.sigmoid(logits.float())
+def route_topk(logits, n_out, top, count=1, keep=1, score="sigmoid", group_score="top2", correction=None, real=None):
+    """Group-limited top-k routing over the first ``n_out`` columns of f32 logits [T, >= n_out].
+    Scores s = sigmoid or softmax of the logits; the choice is made on s + ``correction`` (f32
+    [n_out]).  The outputs form ``count`` groups of neighbours; a group scores the sum of its two best
+    choice scores ("top2") or its best ("max"); the ``top`` best outputs inside the ``keep`` best
+    groups are chosen (ties: the lower index); weights = their scores s as they are.  ``real`` < n_out:
+    the outputs from ``real`` on are identity experts; their weights are summed per token into the
+    third result and left as 0 in the second.  -> ids [T, top] int32, w [T, top] f32, idw [T] f32."""
+    z = logits[:, :n_out].float()
+    s = torch.sigmoid(z) if score == "sigmoid" else torch.softmax(z, -1)
+    ch = s if correction is None else s + correction.float()[None, :]
     T, E = s.shape
     per = E // count
     allowed = torch.ones((T, E), dtype=torch.bool, device=s.device)
     if count > 1 and keep < count:
-        gs = s.view(T, count, per).topk(min(2, per), -1).values.sum(-1)
+        gv = ch.view(T, count, per)
+        gs = gv.topk(min(2, per), -1).values.sum(-1) if group_score == "top2" else gv.max(-1).values
         order = torch.sort(gs, dim=-1, descending=True, stable=True).indices[:, :keep]
         ok = torch.zeros((T, count), dtype=torch.bool, device=s.device)
         ok.scatter_(1, order, True)
         allowed = ok.repeat_interleave(per, 1)
-    masked = torch.where(allowed, s, torch.full_like(s, -1.0))
+    masked = torch.where(allowed, ch, torch.full_like(ch, float("-inf")))
     ids = torch.sort(masked, dim=-1, descending=True, stable=True).indices[:, :top]
-    return ids.to(torch.int32), s.gather(1, ids)
+    w = s.gather(1, ids)
+    idw = torch.zeros(T, dtype=torch.float32, device=s.device)
+    if real is not None and real < n_out:
+        ident = ids >= real
+        idw = torch.where(ident, w, torch.zeros_like(w)).sum(-1)
+        w = torch.where(ident, torch.zeros_like(w), w)
+    return ids.to(torch.int32), w, idw
+
+
+def group_router(logits, top, count, keep):
+    """Sigmoid scores, a group scores the sum of its two best experts, weights = the chosen scores
+    (``route_topk`` with its defaults).  -> ids [T, top] int32, w [T, top] f32."""
+    ids, w, _ = route_topk(logits, logits.shape[1], top, count, keep)
+    return ids, w
 
 
 def swiglu_scale(gu, gate, ff):
@@ -882,3 +915,81 @@ def swiglu_scale(gu, gate, ff):
 def softcap(x, cap):
     """cap * tanh(x / cap) in f32."""
     return cap * torch.tanh(x.float() / cap)
+
+
+# ----------------------------------------------------------------------------- layer-norm layers with layer scale, wide q/k norms, gated activations
+
+def ls_resadd_ln(x, w, b, eps, out_dtype, y=None, ls=None, bias=None, y2=None, g2=None, h=None, hw=None):
+    """The tail of a sublayer of a pre-norm model and the layer norm ahead of the next one:
+    x (f32 stream, in place) += ls * (y + bias + sigmoid(g2) y2 + hw h), every term after y optional
+    (``g2`` and ``hw`` hold one number per token), then returns layernorm(x) * w + b in ``out_dtype``
+    (mean and variance over the row, eps inside the root).  Without y the stream is only normed."""
+    if y is not None:
+        t = y.float()
+        if bias is not None:
+            t = t + bias.float()
+        if y2 is not None:
+            t = t + torch.sigmoid(g2.float()).reshape(-1, 1) * y2.float()
+        if h is not None:
+            t = t + hw.float().reshape(-1, 1) * h.float()
+        x += t if ls is None else t * ls.float()
+    return torch.nn.functional.layer_norm(x, (x.shape[-1],), w.float(), b.float(), eps).to(out_dtype)
+
+
+def proj_norm_prep(proj, heads, kv_heads, dim, vdim, qnorm_w, knorm_w, cos_sin, rot_dims, interleaved, eps, qscale,
+                   vnorm, positions, slots, k_cache, v_cache):
+    """Attention inputs whose q / k norm runs over the whole projection: proj [T, >= heads dim
+    (+ kv_heads dim + kv_heads vdim)] (q | k | v).  q (all heads together) and k (all key heads
+    together) get an RMS norm with weights of that length, then rotary positions on the first
+    ``rot_dims`` dims of every head, pairs (2i, 2i + 1) when ``interleaved`` else (i, i + rot_dims/2);
+    q times ``qscale[head]``.  With ``vnorm`` every value head is divided by its root mean square.
+    k and v go to their page slots (k_cache [blocks, kv_heads, block, dim], v_cache [blocks,
+    kv_heads, vdim, block]); without caches (a layer that reads another layer's) only q is made.
+    Returns q [T, heads, dim]."""
+    T, H, G, d, dv = proj.shape[0], heads, kv_heads, dim, vdim
+    pf = proj.float()
+    half = rot_dims // 2
+    c, s = _rot_table(cos_sin, positions, half) if half > 0 else (None, None)
+
+    def norm_rot(t, w, n):
+        t = (t * torch.rsqrt(t.pow(2).mean(-1, keepdim=True) + eps) * w.float()).reshape(T, n, d).clone()
+        if half > 0:
+            cc, ss = c[:, None, :], s[:, None, :]
+            if interleaved:
+                u, w_ = t[..., 0:rot_dims:2].clone(), t[..., 1:rot_dims:2].clone()
+                t[..., 0:rot_dims:2] = u * cc - w_ * ss
+                t[..., 1:rot_dims:2] = w_ * cc + u * ss
+            else:
+                u, w_ = t[..., :half].clone(), t[..., half:2 * half].clone()
+                t[..., :half] = u * cc - w_ * ss
+                t[..., half:2 * half] = w_ * cc + u * ss
+        return t
+
+    q = norm_rot(pf[:, :H * d], qnorm_w, H) * qscale.float()[None, :, None]
+    if k_cache is not None:
+        k = norm_rot(pf[:, H * d:(H + G) * d], knorm_w, G)
+        v = pf[:, (H + G) * d:(H + G) * d + G * dv].reshape(T, G, dv)
+        if vnorm:
+            v = v * torch.rsqrt(v.pow(2).mean(-1, keepdim=True) + eps)
+        live = slots >= 0
+        sl = slots[live].long()
+        BSz = k_cache.shape[2]
+        k_cache[sl // BSz, :, sl % BSz] = k[live].to(k_cache.dtype)
+        v_cache[sl // BSz, :, :, sl % BSz] = v[live].to(v_cache.dtype)
+    return q.to(proj.dtype)
+
+
+def glu_act(gu, bias=None, mode="swiglu", limit=0.0, alpha=1.0):
+    """gu [T, 2 ff] (gate columns, then up columns), ``bias`` f32 over the same columns -> [T, ff].
+    "swiglu": silu(g) u.  "clamped": g <- min(g, limit), u <- clamp(u, -limit, limit), then
+    g sigmoid(alpha g) (u + 1)."""
+    f = gu.float()
+    if bias is not None:
+        f = f + bias.float()
+    ff = f.shape[1] // 2
+    g, u = f[:, :ff], f[:, ff:]
+    if mode == "swiglu":
+        return (torch.nn.functional.silu(g) * u).to(gu.dtype)
+    g = g.clamp(max=limit)
+    u = u.clamp(min=-limit, max=limit)
+    return (g * torch.sigmoid(alpha * g) * (u + 1.0)).to(gu.dtype)

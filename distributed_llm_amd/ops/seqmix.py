@@ -50,19 +50,21 @@ def norm_resadd(y: torch.Tensor, w: torch.Tensor, eps: float, x: torch.Tensor,
     return x
 
 
-def causal_conv_silu(x, w, b, conv_state, qstart, qlen, ctx, rows, refill: bool = False) -> torch.Tensor:
+def causal_conv_silu(x, w, b, conv_state, qstart, qlen, ctx, rows, refill: bool = False,
+                     act: str = "silu") -> torch.Tensor:
     """``refill``: the step brings at most one token per sequence (a decode step) and the kernel also
     moves each token's input into its slot; otherwise the slot is left to ``conv_state_refill`` or
-    to the scan."""
+    to the scan.  ``act`` "residual": no activation, y = x + the convolution (an input convolution
+    ahead of a mixer)."""
     ext = _native(x)
     if ext is None:
-        y = ref.causal_conv_silu(x, w, b, conv_state, qstart, qlen, ctx, rows)
+        y = ref.causal_conv_silu(x, w, b, conv_state, qstart, qlen, ctx, rows, act)
         if refill:
             ref.conv_state_refill(x, conv_state, qstart, qlen, ctx, rows)
         return y
     # rows of no sequence (graph padding) stay zero, never stale memory
     y = torch.zeros((x.shape[0], w.shape[0]), dtype=x.dtype, device=x.device)
-    ext.causal_conv_silu(x, w, b, conv_state, qstart, qlen, ctx, rows, y, bool(refill))
+    ext.causal_conv_silu(x, w, b, conv_state, qstart, qlen, ctx, rows, y, bool(refill), 0 if act == "silu" else 1)
     return y
 
 
@@ -284,28 +286,31 @@ GQA_SPLIT_TARGET = 512     # workgroups a small matrix-core attention grid is sp
 GQA_SPLIT_MAX = 16
 
 
-def gqa_splits(n_tiles: int, kv_heads: int, max_ctx: int, window: int = 0) -> int:
+def gqa_splits(n_tiles: int, kv_heads: int, max_ctx: int, window: int = 0, keep_first: int = 0) -> int:
     """Key splits of a matrix-core attention launch: grids with few workgroups (decode steps at small
     batch, short portions) split every row's 64-key tiles over up to ``GQA_SPLIT_MAX`` workgroups."""
     tiles = (int(max_ctx) + 63) // 64 if max_ctx > 0 else GQA_SPLIT_MAX     # decode graphs: any context
     if window > 0:
-        tiles = min(tiles, (int(window) + 62) // 64 + 1)
+        tiles = min(tiles, (int(window) + 62) // 64 + 1 + (int(keep_first) + 63) // 64)
     return max(1, min(GQA_SPLIT_MAX, tiles, GQA_SPLIT_TARGET // max(1, n_tiles * kv_heads)))
 
 
 def paged_gqa_attention(q, k_cache, v_cache, block_tables, qstart, qlen, ctx, tile_seq, tile_tok0,
                         gate: Optional[torch.Tensor] = None, mfma: bool = False, splits: int = 1, window: int = 0,
-                        out_f32: bool = False) -> torch.Tensor:
+                        out_f32: bool = False, keep_first: int = 0, sink: float = 0.0) -> torch.Tensor:
     """Causal softmax attention over paged keys / values of any head widths (f32 scores, online
     softmax), output times sigmoid(gate).  ``tile_seq`` / ``tile_tok0``: one entry per
     ``gqa_tokens_per_tile(heads, kv_heads, mfma)`` new tokens of a sequence.  ``splits`` > 1
     (matrix-core kernel): a row's keys are split over that many workgroups and merged.
     ``window`` > 0: a position sees itself and the ``window - 1`` keys before it (older key tiles are
-    not read).  A value cache with fewer heads than the key cache is shared by neighbouring key
-    heads.  ``out_f32``: the output stays f32 whatever the model dtype."""
+    not read), and with ``keep_first`` > 0 also the keys j < keep_first at any distance (their tiles
+    are read as well).  ``sink`` > 0: one more term of score 0 and that weight in every softmax
+    denominator, with no value.  A value cache with fewer heads than the key cache is shared by
+    neighbouring key heads.  ``out_f32``: the output stays f32 whatever the model dtype."""
     ext = _native(q)
     if ext is None:
-        return ref.paged_gqa_attention(q, k_cache, v_cache, block_tables, qstart, qlen, ctx, gate, window, out_f32)
+        return ref.paged_gqa_attention(q, k_cache, v_cache, block_tables, qstart, qlen, ctx, gate, window, out_f32,
+                                       keep_first, sink)
     dv = v_cache.shape[2]
     out = torch.zeros((q.shape[0], q.shape[1] * dv), dtype=torch.float32 if out_f32 else q.dtype, device=q.device)
     splits = int(splits) if mfma else 1
@@ -314,7 +319,7 @@ def paged_gqa_attention(q, k_cache, v_cache, block_tables, qstart, qlen, ctx, ti
         part = torch.empty(int(tile_seq.numel()) * k_cache.shape[1] * splits * GQA_ROWS_MFMA * (dv + 2),
                            dtype=torch.float32, device=q.device)
     ext.paged_gqa_attention(q, k_cache, v_cache, block_tables, qstart, qlen, ctx, tile_seq, tile_tok0, gate, out,
-                            bool(mfma), splits, part, int(window))
+                            bool(mfma), splits, part, int(window), int(keep_first), float(sink))
     return out
 
 
@@ -416,17 +421,34 @@ def polynorm(z: torch.Tensor, coef: torch.Tensor, eps: float) -> torch.Tensor:
     return y
 
 
+def route_topk(logits: torch.Tensor, n_out: int, top: int, count: int = 1, keep: int = 1, score: str = "sigmoid",
+               group_score: str = "top2", correction: Optional[torch.Tensor] = None,
+               real: Optional[int] = None) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """Group-limited top-k routing over the first ``n_out`` columns of f32 logits [T, >= n_out]
+    (further columns, e.g. a gate logit made by the same GEMM, are not read).  Scores s: sigmoid or
+    softmax of the logits; the choice is made on s + ``correction`` (f32 [n_out]); ``count`` groups of
+    neighbouring outputs, a group scores the sum of its two best choice scores ("top2") or its best
+    ("max"); the ``top`` best outputs of the ``keep`` best groups are chosen; weights = their s, not
+    renormalised.  Outputs from ``real`` on are identity experts: their weights are summed per token
+    into ``idw`` and left 0 in ``w`` (the expert kernels then add nothing for them).
+    -> ids [T, top] int32, w [T, top] f32, idw [T] f32."""
+    ext = _native(logits)
+    if ext is None:
+        return ref.route_topk(logits, n_out, top, count, keep, score, group_score, correction, real)
+    T = logits.shape[0]
+    ids = torch.empty((T, top), dtype=torch.int32, device=logits.device)
+    w = torch.empty((T, top), dtype=torch.float32, device=logits.device)
+    idw = torch.empty((T,), dtype=torch.float32, device=logits.device)
+    ext.route_topk(logits, int(n_out), int(top), int(count), int(keep), 0 if score == "sigmoid" else 1,
+                   0 if group_score == "top2" else 1, correction, int(n_out if real is None else real), ids, w, idw)
+    return ids, w, idw
+
+
 def group_router(logits: torch.Tensor, top: int, count: int, keep: int) -> Tuple[torch.Tensor, torch.Tensor]:
     """Sigmoid scores of f32 router logits [T, E]; ``count`` groups of neighbouring experts, a group
     scores the sum of its two best, the ``top`` best experts of the ``keep`` best groups are chosen;
     weights = their scores, not renormalised.  -> ids [T, top] int32, weights [T, top] f32."""
-    ext = _native(logits)
-    if ext is None:
-        return ref.group_router(logits, top, count, keep)
-    T = logits.shape[0]
-    ids = torch.empty((T, top), dtype=torch.int32, device=logits.device)
-    w = torch.empty((T, top), dtype=torch.float32, device=logits.device)
-    ext.group_router(logits, int(top), int(count), int(keep), ids, w)
+    ids, w, _ = route_topk(logits, logits.shape[1], top, count, keep)
     return ids, w
 
 
@@ -493,3 +515,54 @@ def delta_rule(qkv, gba, heads, kv_heads, dim, vdim, neg_a, dt_bias, norm_w, eps
     ext.delta_rule(qkv, gba, int(heads), int(kv_heads), int(dim), int(vdim), neg_a, dt_bias, norm_w, float(eps), state,
                    qstart, qlen, ctx, rows, out)
     return out
+
+
+# ----------------------------------------------------------------------------- layer-norm layers with layer scale, wide q/k norms, gated activations
+
+def ls_resadd_ln(x: torch.Tensor, w: torch.Tensor, b: torch.Tensor, eps: float, out_dtype,
+                 y: Optional[torch.Tensor] = None, ls: Optional[torch.Tensor] = None,
+                 bias: Optional[torch.Tensor] = None, y2: Optional[torch.Tensor] = None,
+                 g2: Optional[torch.Tensor] = None, h: Optional[torch.Tensor] = None,
+                 hw: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """A pre-norm sublayer's tail and the next layer norm in one launch: the f32 stream x [T, width]
+    (in place) += ls * (y + bias + sigmoid(g2) y2 + hw h), every term after y optional (``g2`` f32,
+    one logit per token, may be a column of a wider matrix; ``hw`` f32 [T]); returns
+    layernorm(x) * w + b (mean and variance over the row) in ``out_dtype``.  Without y: the norm alone."""
+    ext = _native(x)
+    if ext is None:
+        return ref.ls_resadd_ln(x, w, b, eps, out_dtype, y, ls, bias, y2, g2, h, hw)
+    out = torch.empty(x.shape, dtype=out_dtype, device=x.device)
+    ext.ls_resadd_ln(x, w, b, float(eps), out, y, ls, bias, y2, g2, h, hw)
+    return out
+
+
+def proj_norm_prep(proj, heads, kv_heads, dim, vdim, qnorm_w, knorm_w, cos_sin, rot_dims, interleaved, eps, qscale,
+                   vnorm, positions, slots, k_cache, v_cache) -> torch.Tensor:
+    """Attention inputs with the q / k RMS norm taken over the whole projection (all heads together,
+    weights of that length) before the rotation; rotary pairs (2i, 2i + 1) when ``interleaved`` else
+    (i, i + rot_dims / 2) on the first ``rot_dims`` dims of every head; q times ``qscale[head]`` (f32);
+    ``vnorm``: every value head to unit RMS.  proj [T, q | k | v]; k and v go to their page slots
+    (k_cache [blocks, kv_heads, block, dim], v_cache [blocks, kv_heads, vdim, block]); ``k_cache``
+    None (a layer that reads another layer's keys and values): proj holds q alone.
+    Returns q [T, heads, dim]."""
+    ext = _native(proj)
+    if ext is None:
+        return ref.proj_norm_prep(proj, heads, kv_heads, dim, vdim, qnorm_w, knorm_w, cos_sin, rot_dims, interleaved,
+                                  eps, qscale, vnorm, positions, slots, k_cache, v_cache)
+    q = torch.empty((proj.shape[0], heads, dim), dtype=proj.dtype, device=proj.device)     # every row is written
+    ext.proj_norm_prep(proj, int(heads), int(kv_heads), int(dim), int(vdim), qnorm_w, knorm_w, cos_sin, int(rot_dims),
+                       bool(interleaved), float(eps), qscale, bool(vnorm), positions, slots, k_cache, v_cache, q)
+    return q
+
+
+def glu_act(gu: torch.Tensor, bias: Optional[torch.Tensor] = None, mode: str = "swiglu", limit: float = 0.0,
+            alpha: float = 1.0) -> torch.Tensor:
+    """Gated activation of gu [T, 2 ff] (gate columns, then up columns; ``bias`` f32 over the same
+    columns) -> [T, ff]: "swiglu" silu(g) u, or "clamped": g <- min(g, limit), u <- clamp(u, -limit,
+    limit), g sigmoid(alpha g) (u + 1)."""
+    ext = _native(gu)
+    if ext is None:
+        return ref.glu_act(gu, bias, mode, limit, alpha)
+    y = torch.empty((gu.shape[0], gu.shape[1] // 2), dtype=gu.dtype, device=gu.device)
+    ext.glu_act(gu, bias, 0 if mode == "swiglu" else 1, float(limit), float(alpha), y)
+    return y
