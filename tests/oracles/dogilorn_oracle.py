@@ -7,8 +7,6 @@ weight and bias, ls a learned vector and canon(h) = h + a short causal convoluti
 Weights come as a dict under the checkpoint's names ('l<i>.mix.<name>', 'l<i>.mlp.<name>'), the
 configuration as the parsed config.json.
 """
-import math
-
 import torch
 
 F64 = torch.float64
@@ -119,7 +117,7 @@ def experts(h, W, p, f):
     """Routed experts; the last ``identity`` router outputs stand for experts that return their
     input.  A shared expert, if any, is added times sigmoid(W_sg h)."""
     r = f["router"]
-    E, ident = r["experts"], r.get("identity", 0)
+    E = r["experts"]
     g = r.get("groups") or {}
     T = h.shape[0]
     z = h @ W[p + "router"].T
@@ -158,48 +156,10 @@ def forward(tokens, W, cfg, taps=None):
     return layer_norm(x, W["final.norm"], W["final.norm.b"], eps) @ W["embed"].T
 
 
-def random_weights(cfg, seed=0):
-    """Random tensors under the checkpoint's names for a parsed config (tests)."""
-    g = torch.Generator().manual_seed(seed)
-    W_, V = cfg["width"], cfg["vocab"]
-    t = {}
-
-    def lin(n_out, n_in, s=1.0):
-        return torch.randn(n_out, n_in, generator=g) * (s / math.sqrt(n_in))
-
-    def vec(n, mean=0.0, s=0.1):
-        return mean + torch.randn(n, generator=g) * s
-
-    t["embed"] = torch.randn(V, W_, generator=g) * 0.5
-    t["final.norm"], t["final.norm.b"] = vec(W_, 1.0), vec(W_)
-    K = cfg["canon"]["taps"]
-    for i, L in enumerate(cfg["layers"]):
-        p, m = f"l{i}.", L["mixer"]
-        for n in ("norm1", "norm2"):
-            t[p + n], t[p + n + ".b"] = vec(W_, 1.0), vec(W_)
-        t[p + "ls1"], t[p + "ls2"] = vec(W_, 0.5, 0.2), vec(W_, 0.5, 0.2)
-        t[p + "canon1"] = torch.randn(W_, K, generator=g) * 0.3
-        H, G, d, dv = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
-        t[p + "mix.q"], t[p + "mix.q.norm"] = lin(H * d, W_), vec(H * d, 1.0, 0.3)
-        t[p + "mix.temp"], t[p + "mix.o"] = vec(H, 1.0, 0.3), lin(W_, H * dv)
-        if m.get("kv_from") is None:
-            t[p + "mix.k"], t[p + "mix.k.norm"] = lin(G * d, W_), vec(G * d, 1.0, 0.3)
-            t[p + "mix.v"] = lin(G * dv, W_)
-        f = L.get("mlp")
-        if not f:
-            del t[p + "norm2"], t[p + "norm2.b"], t[p + "ls2"]
-        elif f["kind"] == "dense":
-            for n, (a, b) in (("gate", (f["ff"], W_)), ("up", (f["ff"], W_)), ("down", (W_, f["ff"]))):
-                t[p + "mlp." + n], t[p + "mlp." + n + ".b"] = lin(a, b, 2.0), vec(a, 0.0, 0.3)
-        else:
-            r = f["router"]
-            R = r["experts"] + r.get("identity", 0)
-            t[p + "mlp.router"], t[p + "mlp.correction"] = lin(R, W_, 2.0), vec(R, 0.0, 0.05)
-            names = [f"e{e}" for e in range(r["experts"])] + (["shared"] if f.get("shared") else [])
-            for n in names:
-                ff = f["shared"]["ff"] if n == "shared" else f["expert"]["ff"]
-                t[p + f"mlp.{n}.gate"], t[p + f"mlp.{n}.up"] = lin(ff, W_), lin(ff, W_)
-                t[p + f"mlp.{n}.down"] = lin(W_, ff)
-            if f.get("shared"):
-                t[p + "mlp.shared.sg"] = lin(1, W_)
-    return {k: v.to(torch.bfloat16) for k, v in t.items()}
+def greedy(tokens, W, cfg, n):
+    """n arg-max continuations of a prompt (the whole sequence is recomputed for every token)."""
+    seq, out = list(tokens), []
+    for _ in range(n):
+        out.append(int(forward(seq, W, cfg)[-1].argmax()))
+        seq.append(out[-1])
+    return out

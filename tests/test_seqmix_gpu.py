@@ -484,3 +484,116 @@ def test_group_router(E, top, count, keep):
     i2, w2 = ref.group_router(logits, top, count, keep)
     assert torch.equal(i1, i2)
     torch.testing.assert_close(w1, w2, atol=1e-6, rtol=1e-6)
+
+
+# ----------------------------------------------------------------------------- layer-norm layers, input convolution, wide q/k norms, sink attention
+
+@pytest.mark.parametrize("dt", DTYPES)
+@pytest.mark.parametrize("n", [24, 104, 328, 1000])
+@pytest.mark.parametrize("terms", ["none", "y", "y+bias", "all", "all-no-gate"])
+def test_ls_resadd_ln(dt, n, terms):
+    torch.manual_seed(21)
+    T = 11
+    x1 = torch.randn(T, n, device=DEV) * 3 + 0.7
+    x2 = x1.clone()
+    w, b, ls, bias = (torch.randn(n, device=DEV) for _ in range(4))
+    kw = {}
+    if terms != "none":
+        kw = dict(y=torch.randn(T, n + 3, device=DEV).to(dt)[:, :n], ls=ls)
+    if terms in ("y+bias", "all"):
+        kw["bias"] = bias
+    if terms.startswith("all"):
+        z = torch.randn(T, 5, device=DEV)
+        kw.update(y2=torch.randn(T, n, device=DEV).to(dt), h=torch.randn(T, n, device=DEV).to(dt), hw=torch.rand(T, device=DEV))
+        if terms == "all":
+            kw["g2"] = z[:, 3]      # a column of a wider matrix
+    got = seqmix.ls_resadd_ln(x1, w, b, 1e-5, dt, **kw)
+    want = ref.ls_resadd_ln(x2, w, b, 1e-5, dt, **kw)
+    torch.testing.assert_close(x1, x2, atol=1e-5, rtol=1e-5)
+    torch.testing.assert_close(got.float(), want.float(), **tol(dt))
+
+
+@pytest.mark.parametrize("dt", DTYPES)
+@pytest.mark.parametrize("case", CASES)
+@pytest.mark.parametrize("C,K", [(40, 3), (128, 4), (72, 1), (64, 7)])
+def test_input_convolution(dt, case, C, K):
+    """y = x + conv(x) without an activation; decode steps refill the slot in the same launch."""
+    torch.manual_seed(22)
+    T, qstart, qlen, ctx, rows, pos = batch(*case)
+    x = torch.randn(T, C + 5, device=DEV).to(dt)
+    w, b = torch.randn(C, K, device=DEV) * 0.5, torch.zeros(C, device=DEV)
+    st1 = torch.randn(len(case[0]), K - 1, C, device=DEV).to(dt)
+    st2 = st1.clone()
+    single = max(case[0]) <= 1
+    got = seqmix.causal_conv_silu(x, w, b, st1, qstart, qlen, ctx, rows, refill=single, act="residual")
+    want = ref.causal_conv_silu(x, w, b, st2, qstart, qlen, ctx, rows, act="residual")
+    torch.testing.assert_close(got.float(), want.float(), **tol(dt))
+    if not single:
+        seqmix.conv_state_refill(x, st1, qstart, qlen, ctx, rows)
+    ref.conv_state_refill(x, st2, qstart, qlen, ctx, rows)
+    torch.testing.assert_close(st1.float(), st2.float(), atol=0, rtol=0)
+
+
+@pytest.mark.parametrize("dt", DTYPES)
+def test_glu_act(dt):
+    torch.manual_seed(23)
+    gu = (torch.randn(33, 2 * 70 + 4, device=DEV) * 3).to(dt)[:, :140]
+    bias = torch.randn(140, device=DEV)
+    for kw in (dict(), dict(bias=bias), dict(bias=bias, mode="clamped", limit=1.5, alpha=1.702), dict(mode="clamped", limit=0.3, alpha=1.0)):
+        torch.testing.assert_close(seqmix.glu_act(gu, **kw).float(), ref.glu_act(gu, **kw).float(), **tol(dt))
+
+
+@pytest.mark.parametrize("score", ["softmax", "sigmoid"])
+@pytest.mark.parametrize("group_score", ["max", "top2"])
+@pytest.mark.parametrize("R,real,top,count,keep", [(16, 12, 3, 2, 1), (16, 16, 4, 1, 1), (12, 7, 3, 4, 2), (64, 60, 8, 8, 3), (5, 0, 5, 5, 5),
+                                                   (6, 5, 1, 6, 1), (200, 190, 6, 4, 4)])
+def test_route_topk(score, group_score, R, real, top, count, keep):
+    torch.manual_seed(24)
+    logits = torch.randn(37, R + 2, device=DEV) * 2
+    for corr in (None, torch.randn(R, device=DEV) * 0.3 - 0.2):
+        a = seqmix.route_topk(logits, R, top, count, keep, score, group_score, corr, real)
+        b = ref.route_topk(logits, R, top, count, keep, score, group_score, corr, real)
+        assert torch.equal(a[0], b[0])
+        torch.testing.assert_close(a[1], b[1], atol=1e-6, rtol=1e-5)
+        torch.testing.assert_close(a[2], b[2], atol=1e-6, rtol=1e-5)
+        assert bool(((a[0] >= real) == (a[1] == 0)).all())
+
+
+@pytest.mark.parametrize("dt", DTYPES)
+@pytest.mark.parametrize("case", CASES + [([40, 3], [90, 130]), ([1, 1], [300, 77]), ([150], [170])])
+@pytest.mark.parametrize("H,G,d,dv,rot,win,keep", [(4, 2, 16, 8, 8, 5, 3), (6, 2, 88, 56, 20, 64, 70), (3, 3, 40, 72, 40, 1, 0),
+                                                   (8, 1, 96, 96, 24, 100, 20), (4, 1, 56, 88, 28, 70, 1), (2, 1, 136, 200, 64, 0, 9),
+                                                   (5, 5, 24, 40, 0, 17, 130), (8, 2, 64, 64, 64, 3, 64)])
+def test_sink_attention_kernels(dt, case, H, G, d, dv, rot, win, keep):
+    """Prep (norm over the whole q / k projection before an interleaved rotation, unit-RMS values),
+    then attention with a window, kept first keys and a sink, in both kernel forms and every split
+    count; a layer that reads another layer's pages makes the same queries."""
+    from distributed_llm_amd.models.llama import AttnMeta
+    torch.manual_seed(25)
+    T, qstart, qlen, ctx, pos, bt, kc, vc, slots = _pages(case, G, d, dv, dt)
+    cols = H * d + G * (d + dv)
+    proj = torch.randn(T, cols + 3, device=DEV).to(dt)
+    qw, kw = torch.rand(H * d, device=DEV) + 0.5, torch.rand(G * d, device=DEV) + 0.5
+    qscale = torch.rand(H, device=DEV) * 0.6 + 0.2
+    table = ops.rope_cos_sin(512, max(rot, 2), 100.0, DEV)
+    for inter in (True, False):
+        kc2, vc2 = kc.clone(), vc.clone()
+        kc1, vc1 = kc.clone(), vc.clone()
+        q1 = seqmix.proj_norm_prep(proj, H, G, d, dv, qw, kw, table, rot, inter, 1e-5, qscale, inter, pos, slots, kc1, vc1)
+        q2 = ref.proj_norm_prep(proj, H, G, d, dv, qw, kw, table, rot, inter, 1e-5, qscale, inter, pos, slots, kc2, vc2)
+        torch.testing.assert_close(q1.float(), q2.float(), **tol(dt))
+        torch.testing.assert_close(kc1.float(), kc2.float(), **tol(dt))
+        torch.testing.assert_close(vc1.float(), vc2.float(), **tol(dt))
+        q3 = seqmix.proj_norm_prep(proj, H, G, d, dv, qw, qw, table, rot, inter, 1e-5, qscale, inter, pos, slots, None, None)
+        torch.testing.assert_close(q3.float(), q2.float(), **tol(dt))
+    meta = AttnMeta(slots=None, block_tables=bt, qstart=qstart, qlen=qlen, ctx=ctx, tile_seq=None, tile_tok0=None,
+                    last_idx=None, host_qlen=case[0])
+    forms = [False] + ([True] if seqmix.gqa_use_mfma(q2, H, G, d, dv, 16) else [])
+    for sink in (1.0, 0.0):
+        want = ref.paged_gqa_attention(q2, kc2, vc2, bt, qstart, qlen, ctx, None, win, False, keep, sink).float()
+        for mfma in forms:
+            ts, tt = meta.latent_tiles(1, DEV, seqmix.gqa_tokens_per_tile(H, G, mfma))
+            for splits in ((1, 2, 7) if mfma else (1,)):
+                got = seqmix.paged_gqa_attention(q2, kc2, vc2, bt, qstart, qlen, ctx, ts, tt, None, mfma, splits, window=win,
+                                                 keep_first=keep, sink=sink).float()
+                torch.testing.assert_close(got, want, **tol(dt))
