@@ -929,7 +929,7 @@ def ls_resadd_ln(x, w, b, eps, out_dtype, y=None, ls=None, bias=None, y2=None, g
         if bias is not None:
             t = t + bias.float()
         if y2 is not None:
-            t = t + torch.sigmoid(g2.float()).reshape(-1, 1) * y2.float()
+            t = t + (y2.float() if g2 is None else torch.sigmoid(g2.float()).reshape(-1, 1) * y2.float())
         if h is not None:
             t = t + hw.float().reshape(-1, 1) * h.float()
         x += t if ls is None else t * ls.float()
