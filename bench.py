@@ -110,7 +110,7 @@ def parse():
                          "Llama-family model at equal size, prefill / decode throughput and mixer-kernel rooflines "
                          "(prints its own JSON object)")
     ap.add_argument("--arch-size", default="s", choices=["s", "m"])
-    ap.add_argument("--arch-design", default="filevik", choices=["filevik", "sedopel", "pebodra"],
+    ap.add_argument("--arch-design", default="filevik", choices=["filevik", "sedopel", "pebodra", "dogilorn"],
                     help="with --arch-bench: which layer-list design runs beside its closest Llama-family model")
     ap.add_argument("--arch-kernels-only", action="store_true")
     ap.add_argument("--trace", default=None,

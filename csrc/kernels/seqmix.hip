@@ -764,6 +764,7 @@ __global__ void __launch_bounds__(256) route_topk_kernel(const float* __restrict
         if (!ok[g] && (v > bv || bi == 0x7fffffff)) { bv = v; bi = g; }
       }
       wave_argmax(bv, bi);
+      if (bi == 0x7fffffff) bi = 0;
       if (lane == 0) ok[bi] = 1;
       __builtin_amdgcn_wave_barrier();
     }
@@ -777,6 +778,7 @@ __global__ void __launch_bounds__(256) route_topk_kernel(const float* __restrict
       if (v > bv && (!limited || ok[e / per])) { bv = v; bi = e; }
     }
     wave_argmax(bv, bi);
+    if (bi == 0x7fffffff) bi = 0;     // a row of NaNs (stale padding) compares false everywhere: stay inside the arrays
     if (lane == 0) {
       const float w = sc[bi];
       ids[(long)t * top + j] = bi;

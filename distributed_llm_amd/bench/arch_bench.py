@@ -1,9 +1,18 @@
-"""Layer-list (Filevik, Sedopel, Pebodra) models beside the closest Llama-family model at equal size:
+"""Layer-list (Filevik, Sedopel, Pebodra, Dogilorn) models beside the closest Llama-family model at equal size:
 prefill and decode throughput through the engine, and the time of each mixer kernel against its roofline.
 
-``python bench.py --arch-bench [--arch-design filevik|sedopel|pebodra] [--arch-size s|m]`` (random
+``python bench.py --arch-bench [--arch-design filevik|sedopel|pebodra|dogilorn] [--arch-size s|m]`` (random
 weights, synthetic tokens).  The default bench workload and its JSON line are untouched; this prints one
 JSON object of its own.
+
+The Dogilorn stack is attention only (grouped-query, an RMS norm over the whole q and k projections,
+a sliding window that also keeps the first tokens, a sink term in the softmax; every third layer reads
+the keys and values of the layer before it), behind an input convolution and layer norms; its
+feed-forwards alternate between a dense clamped GLU and routed SwiGLU experts with identity experts
+and a gated shared expert.  Its comparison model is the Mixtral-style Llama of the same width, depth
+and experts, and kernel by kernel: attention against the Pebodra and Sedopel attention (the same
+kernels with other options) and the Llama kernels at the same heads, its prep, convolution, residual
+and router launches against the like launches of the other designs.
 
 The Sedopel stack alternates parallel layers (grouped-query softmax attention beside lightning
 attention, dense GELU feed-forward) and gated-delta-rule layers without a feed-forward; its
@@ -62,6 +71,104 @@ PEBODRA_SIZES = {
               state=128, groups=8, conv=4, norm_groups=8, x_heads=16, x_dim=128, x_vdim=128, experts=8, top=2, ff=2048,
               dense_ff=8192, vocab=32000),
 }
+
+
+DOGILORN_SIZES = {
+    "s": dict(width=1024, layers=6, heads=16, kv_heads=4, dim=64, vdim=64, rot=32, window=1024, keep_first=64, taps=4,
+              experts=8, identity=2, top=2, ff=1024, shared=1024, dense_ff=4096, vocab=32000),
+    "m": dict(width=2048, layers=12, heads=16, kv_heads=4, dim=128, vdim=128, rot=64, window=1024, keep_first=128, taps=4,
+              experts=8, identity=2, top=2, ff=2048, shared=2048, dense_ff=8192, vocab=32000),
+}
+
+
+def dogilorn_raw(z: dict) -> dict:
+    moe = {"kind": "moe", "expert": {"ff": z["ff"]}, "shared": {"ff": z["shared"]},
+           "router": {"experts": z["experts"], "identity": z["identity"], "top": z["top"], "groups": {"count": 2, "keep": 1}}}
+    att = {"heads": z["heads"], "kv_heads": z["kv_heads"], "dim": z["dim"], "vdim": z["vdim"], "scale": z["dim"] ** -0.5 * 4.0,
+           "mask": {"size": z["window"], "keep_first": z["keep_first"]}, "rot": {"dims": z["rot"], "base": 10000.0}}
+    layers = []
+    for i in range(z["layers"]):
+        L = {"type": "attention", "mixer": dict(att, kv_from=i - 1) if i % 3 == 2 else dict(att)}
+        L["mlp"] = {"kind": "dense", "ff": z["dense_ff"], "limit": 7.0} if i % 2 == 0 else moe
+        layers.append(L)
+    return {"architecture": "Dogilorn", "width": z["width"], "vocab": z["vocab"], "norm": {"eps": 1e-5},
+            "canon": {"taps": z["taps"]}, "embedding": {"scale": 1.0}, "layers": layers}
+
+
+def dogilorn_kernel_rooflines(z: dict, T: int = 4096, B: int = 64, ctx: int = 2048) -> Dict[str, dict]:
+    """Each Dogilorn kernel alone (bf16): prefill of one T-token sequence, decode of B sequences at
+    ``ctx``; time, the bound resource's minimum time, and their ratio."""
+    from .. import ops
+    from ..models.llama import AttnMeta
+    from ..ops import seqmix
+    dev, bf = "cuda", torch.bfloat16
+    i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=dev)
+    res: Dict[str, dict] = {}
+
+    def rec(name, sec, bytes_, flops, peak_flops):
+        floor = max(bytes_ / PEAK_BW, flops / peak_flops)
+        res[name] = {"us": round(sec * 1e6, 1), "roofline_us": round(floor * 1e6, 2), "x_roofline": round(sec / floor, 1),
+                     "bound": "memory" if bytes_ / PEAK_BW >= flops / peak_flops else "compute"}
+
+    W = z["width"]
+    for tag, qlens, starts in (("prefill", [T], [0]), ("decode", [1] * B, [ctx] * B)):
+        n, S = sum(qlens), len(qlens)
+        qstart = i32([sum(qlens[:i]) for i in range(S)])
+        cxl = [a + b for a, b in zip(starts, qlens)]
+        qlen, cx, rows = i32(qlens), i32(cxl), i32(list(range(S)))
+        pos = i32([p for a, m in zip(starts, qlens) for p in range(a, a + m)])
+        H, G, d, dv, Wn, Kf = z["heads"], z["kv_heads"], z["dim"], z["vdim"], z["window"], z["keep_first"]
+        see = lambda p: min(p + 1, Wn) + max(0, min(Kf, p + 1 - Wn))       # keys position p sees
+        pairs = sum(see(p) for a, m in zip(starts, qlens) for p in range(a, a + m))
+        seen = sum(min(c, Wn + m - 1 + Kf) for c, m in zip(cxl, qlens))    # keys any row of a sequence sees
+        nb = (max(cxl) + 15) // 16
+        bt = torch.arange(S * nb, dtype=torch.int32, device=dev).view(S, nb)
+        kc = (torch.randn(S * nb, G, 16, d, device=dev) * 0.3).to(bf)
+        vc = (torch.randn(S * nb, G, dv, 16, device=dev) * 0.3).to(bf)
+        cols = H * d + G * (d + dv)
+        proj = torch.randn(n, cols, device=dev).to(bf)
+        table = ops.rope_cos_sin(ctx + T + 8, z["rot"], 10000.0, dev)
+        slots = i32([int(bt[i, p // 16]) * 16 + p % 16 for i, (a, m) in enumerate(zip(starts, qlens)) for p in range(a, a + m)])
+        qw, kw, qs = torch.ones(H * d, device=dev), torch.ones(G * d, device=dev), torch.full((H,), d ** -0.5, device=dev)
+        prep = lambda: seqmix.proj_norm_prep(proj, H, G, d, dv, qw, kw, table, z["rot"], True, 1e-5, qs, True, pos, slots, kc, vc)
+        q = prep()
+        rec(f"proj_norm_prep_{tag}", _timed(prep), n * cols * 4, n * cols * 10, PEAK_F32)
+        meta = AttnMeta(slots=None, block_tables=bt, qstart=qstart, qlen=qlen, ctx=cx, tile_seq=None, tile_tok0=None,
+                        last_idx=None, host_qlen=qlens)
+        mfma = seqmix.gqa_use_mfma(q, H, G, d, dv, 16)
+        ts, tt = meta.latent_tiles(1, dev, seqmix.gqa_tokens_per_tile(H, G, mfma))
+        sp = seqmix.gqa_splits(int(ts.numel()), G, max(cxl), Wn, Kf) if mfma else 1
+        att = lambda: seqmix.paged_gqa_attention(q, kc, vc, bt, qstart, qlen, cx, ts, tt, None, mfma, sp, window=Wn,
+                                                 keep_first=Kf, sink=1.0)
+        att()
+        rec(f"attention_{tag}", _timed(att, 3), seen * G * (d + dv) * 2 + n * H * (d + dv) * 2, pairs * H * 2 * (d + dv), PEAK_BF16)
+        # input convolution (h + conv(h)) and its slot
+        K = z["taps"]
+        h = torch.randn(n, W, device=dev).to(bf)
+        cw, cb, cs_ = torch.randn(W, K, device=dev) * 0.3, torch.zeros(W, device=dev), torch.zeros(S, K - 1, W, device=dev, dtype=bf)
+        single = tag == "decode"
+        rec(f"input_conv_{tag}",
+            _timed(lambda: seqmix.causal_conv_silu(h, cw, cb, cs_, qstart, qlen, cx, rows, refill=single, act="residual")),
+            n * W * 4 + (S * (K - 1) * W * 4 if single else 0), n * W * 2 * K, PEAK_F32)
+        # sublayer tail + layer norm (with the expert terms), gated activation, router
+        x = torch.randn(n, W, device=dev)
+        y, y2 = torch.randn(n, W, device=dev).to(bf), torch.randn(n, W, device=dev).to(bf)
+        lw, lb, ls = torch.ones(W, device=dev), torch.zeros(W, device=dev), torch.full((W,), 0.5, device=dev)
+        R = z["experts"] + z["identity"]
+        logits = torch.randn(n, R + 1, device=dev)
+        hw = torch.rand(n, device=dev)
+        rec(f"ls_resadd_ln_{tag}", _timed(lambda: seqmix.ls_resadd_ln(x, lw, lb, 1e-5, bf, y=y, ls=ls)),
+            n * W * (8 + 2 + 2), n * W * 10, PEAK_F32)
+        rec(f"ls_resadd_ln_experts_{tag}",
+            _timed(lambda: seqmix.ls_resadd_ln(x, lw, lb, 1e-5, bf, y=y, ls=ls, y2=y2, g2=logits[:, R], h=h, hw=hw)),
+            n * W * (8 + 2 + 2 + 4), n * W * 14, PEAK_F32)
+        gu, gb = torch.randn(n, 2 * z["dense_ff"], device=dev).to(bf), torch.zeros(2 * z["dense_ff"], device=dev)
+        rec(f"glu_act_{tag}", _timed(lambda: seqmix.glu_act(gu, gb, "clamped", 7.0, 1.702)),
+            n * z["dense_ff"] * 6, n * z["dense_ff"] * 12, PEAK_F32)
+        corr = torch.zeros(R, device=dev)
+        rec(f"route_topk_{tag}", _timed(lambda: seqmix.route_topk(logits, R, z["top"], 2, 1, "softmax", "max", corr, z["experts"])),
+            n * (R + 1) * 4 + n * z["top"] * 8, n * R * 20, PEAK_F32)
+    return res
 
 
 def pebodra_raw(z: dict) -> dict:
@@ -432,7 +539,27 @@ def llama_kernel_rooflines(T: int = 4096, B: int = 64, ctx: int = 2048, nq: int 
 
 
 def run(size: str = "s", kernels_only: bool = False, design: str = "filevik") -> dict:
-    from ..models.configs import filevik_config, pebodra_config, sedopel_config
+    from ..models.configs import dogilorn_config, filevik_config, pebodra_config, sedopel_config
+    if design == "dogilorn":
+        z = DOGILORN_SIZES[size]
+        out = {"bench": "arch", "design": design, "size": size, "dtype": "bf16", "data": "synthetic", "sizes": z}
+        out["dogilorn_kernels"] = dogilorn_kernel_rooflines(z)
+        # the like kernels at like sizes: windowed attention with two maps (Pebodra) and plain grouped-query
+        # attention (Sedopel) at the same score rows and head widths, the Llama attention kernels at the
+        # same heads, and the other designs' prep, convolution and residual launches
+        pz = dict(PEBODRA_SIZES[size], heads=z["heads"] // 2, kv_heads=max(1, z["kv_heads"] // 2), dim=z["dim"], vdim=z["vdim"],
+                  window=z["window"])
+        out["pebodra_kernels"] = pebodra_kernel_rooflines(pz)
+        out["sedopel_kernels"] = sedopel_kernel_rooflines(dict(SEDOPEL_SIZES[size], heads=z["heads"], kv_heads=z["kv_heads"],
+                                                               dim=z["dim"], vdim=z["vdim"]))
+        out["llama_kernels"] = llama_kernel_rooflines(nq=z["heads"], nkv=z["kv_heads"], d=z["dim"])
+        if not kernels_only:
+            prompts, batches = [512, 2048], [1, 16, 64]
+            out["dogilorn"] = engine_throughput(dogilorn_config(dogilorn_raw(z), name=f"dogilorn-{size}"), prompts, batches,
+                                                ctx=1024, new=32, rows=64)
+            out["moe_llama"] = engine_throughput(pebodra_twin(z), prompts, batches, ctx=1024, new=32, rows=64)
+        print(json.dumps(out))
+        return out
     if design == "pebodra":
         z = PEBODRA_SIZES[size]
         out = {"bench": "arch", "design": design, "size": size, "dtype": "bf16", "data": "synthetic", "sizes": z}

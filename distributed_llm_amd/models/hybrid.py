@@ -642,7 +642,7 @@ class HybridModel:
         the sequence's last inputs."""
         single = meta.host_qlen is None      # a decode step: the convolution refills its slots itself
         y = seqmix.causal_conv_silu(h, L["canon"], L["canon_b"], state, meta.qstart, meta.qlen, meta.ctx,
-                                    meta.state_rows, refill=single, act="residual")
+                                    meta.state_rows, refill=single, act="residual", all_rows=self._all_rows(h, meta))
         if not single:
             seqmix.conv_state_refill(h, state, meta.qstart, meta.qlen, meta.ctx, meta.state_rows)
         return y
@@ -660,8 +660,14 @@ class HybridModel:
         ts, tt = meta.latent_tiles(1, self.device, seqmix.gqa_tokens_per_tile(m.heads, m.kv_heads, mfma))
         splits = seqmix.gqa_splits(int(ts.numel()), m.kv_heads, meta.max_ctx, m.window, m.keep_first) if mfma else 1
         o = seqmix.paged_gqa_attention(q, k_cache, v_cache, meta.block_tables, meta.qstart, meta.qlen, meta.ctx, ts, tt,
-                                       None, mfma, splits, window=m.window, keep_first=m.keep_first, sink=m.sink)
+                                       None, mfma, splits, window=m.window, keep_first=m.keep_first, sink=m.sink,
+                                       all_rows=self._all_rows(x, meta))
         return _mm(o, L["o"])
+
+    @staticmethod
+    def _all_rows(x, meta) -> bool:
+        """A step of prompt portions whose sequences cover every packed row (no padding rows)."""
+        return meta.host_qlen is not None and sum(int(n) for n in meta.host_qlen) == x.shape[0]
 
     def _mamba2(self, L, m: MixerSpec, x, meta, cache):
         conv_state, state = cache

@@ -51,11 +51,12 @@ def norm_resadd(y: torch.Tensor, w: torch.Tensor, eps: float, x: torch.Tensor,
 
 
 def causal_conv_silu(x, w, b, conv_state, qstart, qlen, ctx, rows, refill: bool = False,
-                     act: str = "silu") -> torch.Tensor:
+                     act: str = "silu", all_rows: bool = False) -> torch.Tensor:
     """``refill``: the step brings at most one token per sequence (a decode step) and the kernel also
     moves each token's input into its slot; otherwise the slot is left to ``conv_state_refill`` or
     to the scan.  ``act`` "residual": no activation, y = x + the convolution (an input convolution
-    ahead of a mixer)."""
+    ahead of a mixer).  ``all_rows``: every row of x belongs to a sequence (a step of prompt portions
+    without padding), so the output needs no zero fill."""
     ext = _native(x)
     if ext is None:
         y = ref.causal_conv_silu(x, w, b, conv_state, qstart, qlen, ctx, rows, act)
@@ -63,7 +64,7 @@ def causal_conv_silu(x, w, b, conv_state, qstart, qlen, ctx, rows, refill: bool 
             ref.conv_state_refill(x, conv_state, qstart, qlen, ctx, rows)
         return y
     # rows of no sequence (graph padding) stay zero, never stale memory
-    y = torch.zeros((x.shape[0], w.shape[0]), dtype=x.dtype, device=x.device)
+    y = (torch.empty if all_rows else torch.zeros)((x.shape[0], w.shape[0]), dtype=x.dtype, device=x.device)
     ext.causal_conv_silu(x, w, b, conv_state, qstart, qlen, ctx, rows, y, bool(refill), 0 if act == "silu" else 1)
     return y
 
@@ -297,7 +298,8 @@ def gqa_splits(n_tiles: int, kv_heads: int, max_ctx: int, window: int = 0, keep_
 
 def paged_gqa_attention(q, k_cache, v_cache, block_tables, qstart, qlen, ctx, tile_seq, tile_tok0,
                         gate: Optional[torch.Tensor] = None, mfma: bool = False, splits: int = 1, window: int = 0,
-                        out_f32: bool = False, keep_first: int = 0, sink: float = 0.0) -> torch.Tensor:
+                        out_f32: bool = False, keep_first: int = 0, sink: float = 0.0,
+                        all_rows: bool = False) -> torch.Tensor:
     """Causal softmax attention over paged keys / values of any head widths (f32 scores, online
     softmax), output times sigmoid(gate).  ``tile_seq`` / ``tile_tok0``: one entry per
     ``gqa_tokens_per_tile(heads, kv_heads, mfma)`` new tokens of a sequence.  ``splits`` > 1
@@ -306,13 +308,15 @@ def paged_gqa_attention(q, k_cache, v_cache, block_tables, qstart, qlen, ctx, ti
     not read), and with ``keep_first`` > 0 also the keys j < keep_first at any distance (their tiles
     are read as well).  ``sink`` > 0: one more term of score 0 and that weight in every softmax
     denominator, with no value.  A value cache with fewer heads than the key cache is shared by
-    neighbouring key heads.  ``out_f32``: the output stays f32 whatever the model dtype."""
+    neighbouring key heads.  ``out_f32``: the output stays f32 whatever the model dtype.  ``all_rows``:
+    the tiles cover every row of q (no padding rows), so the output needs no zero fill."""
     ext = _native(q)
     if ext is None:
         return ref.paged_gqa_attention(q, k_cache, v_cache, block_tables, qstart, qlen, ctx, gate, window, out_f32,
                                        keep_first, sink)
     dv = v_cache.shape[2]
-    out = torch.zeros((q.shape[0], q.shape[1] * dv), dtype=torch.float32 if out_f32 else q.dtype, device=q.device)
+    out = (torch.empty if all_rows else torch.zeros)((q.shape[0], q.shape[1] * dv),
+                                                     dtype=torch.float32 if out_f32 else q.dtype, device=q.device)
     splits = int(splits) if mfma else 1
     part = None
     if splits > 1:
