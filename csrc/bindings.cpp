@@ -56,7 +56,7 @@ int dllm_ls_resadd_ln(const void*, long, int, const float*, const float*, const 
                       const float*, float*, const float*, const float*, void*, long, int, float, hipStream_t);
 int dllm_glu_act(const void*, long, int, const float*, int, int, float, float, void*, long, hipStream_t);
 int dllm_proj_norm_prep(const void*, long, int, int, int, int, int, const float*, const float*, const float*, int, int, int, float,
-                        const float*, int, const int*, const int*, void*, void*, void*, long, int, hipStream_t);
+                        const float*, int, const int*, const int*, void*, void*, void*, long, int, void*, int, hipStream_t);
 int dllm_group_router(const float*, int, int, int, int, int, int*, float*, hipStream_t);
 int dllm_swiglu_scale(const void*, int, const float*, int, int, void*, long, hipStream_t);
 int dllm_softcap(const void*, int, float, float*, long, hipStream_t);
@@ -1403,6 +1403,8 @@ void causal_conv_silu(torch::Tensor x, torch::Tensor w, torch::Tensor b, torch::
   TORCH_CHECK(y.is_cuda() && y.scalar_type() == x.scalar_type() && y.is_contiguous() && y.dim() == 2 && y.size(0) == T &&
                   y.size(1) == C,
               "y [T, C]");
+  TORCH_CHECK(y.data_ptr() != x.data_ptr() || (refill && x.stride(0) == C),
+              "in place only for steps of single tokens (refill) over exactly the convolved columns");
   auto m = seq_meta(qstart, qlen, ctx, rows, state.size(0));
   ok(dllm_conv_silu(x.data_ptr(), x.stride(0), f, w.data_ptr<float>(), b.data_ptr<float>(), state.data_ptr(), m.qstart,
                     m.qlen, m.ctx, m.rows, y.data_ptr(), T, m.S, C, K, (int)refill, (int)act, stream()),
@@ -1993,11 +1995,20 @@ void glu_act(torch::Tensor gu, c10::optional<torch::Tensor> bias, int64_t mode, 
 void proj_norm_prep(torch::Tensor proj, int64_t H, int64_t G, int64_t d, int64_t dv, torch::Tensor qw, torch::Tensor kw,
                     torch::Tensor cos_sin, int64_t rot, bool interleaved, double eps, torch::Tensor qscale, bool vnorm,
                     torch::Tensor pos, torch::Tensor slots, c10::optional<torch::Tensor> kc, c10::optional<torch::Tensor> vc,
-                    torch::Tensor q) {
+                    torch::Tensor q, c10::optional<torch::Tensor> zero_rows) {
   const bool f = act_f32(proj, "proj");
   check_rows2d(proj, "proj");
   check_f32(cos_sin, "cos_sin");
   check_f32(qw, "q norm weight");
+  void* zp = nullptr;
+  int zn = 0;
+  if (zero_rows) {
+    TORCH_CHECK(zero_rows->is_cuda() && zero_rows->scalar_type() == proj.scalar_type() && zero_rows->is_contiguous() &&
+                    zero_rows->dim() == 2 && zero_rows->size(0) == proj.size(0),
+                "zero_rows [T, n] contiguous in the activations' dtype");
+    zp = zero_rows->data_ptr();
+    zn = (int)zero_rows->size(1);
+  }
   check_f32(kw, "k norm weight");
   check_f32(qscale, "q scale");
   check_i32(pos, "positions");
@@ -2030,7 +2041,7 @@ void proj_norm_prep(torch::Tensor proj, int64_t H, int64_t G, int64_t d, int64_t
   ok(dllm_proj_norm_prep(proj.data_ptr(), proj.stride(0), f, (int)H, (int)G, (int)d, (int)dv, qw.data_ptr<float>(),
                          kw.data_ptr<float>(), cos_sin.data_ptr<float>(), (int)cos_sin.size(1), (int)rot, (int)interleaved,
                          (float)eps, qscale.data_ptr<float>(), (int)vnorm, pos.data_ptr<int>(), slots.data_ptr<int>(), kp, vp,
-                         q.data_ptr(), (long)T, bsz, stream()),
+                         q.data_ptr(), (long)T, bsz, zp, zn, stream()),
      "proj_norm_prep");
 }
 
@@ -2148,7 +2159,10 @@ PYBIND11_MODULE(_hip_kernels, m) {
   m.def("route_topk", &route_topk);
   m.def("ls_resadd_ln", &ls_resadd_ln);
   m.def("glu_act", &glu_act);
-  m.def("proj_norm_prep", &proj_norm_prep);
+  m.def("proj_norm_prep", &proj_norm_prep, py::arg("proj"), py::arg("heads"), py::arg("kv_heads"), py::arg("dim"), py::arg("vdim"),
+        py::arg("qw"), py::arg("kw"), py::arg("cos_sin"), py::arg("rot"), py::arg("interleaved"), py::arg("eps"), py::arg("qscale"),
+        py::arg("vnorm"), py::arg("pos"), py::arg("slots"), py::arg("k_cache"), py::arg("v_cache"), py::arg("q"),
+        py::arg("zero_rows") = py::none());
   m.def("softcap", &softcap);
   m.def("gated_group_norm", &gated_group_norm);
   m.def("outer_scan_cols", []() { return dllm_outer_scan_cols(); });

@@ -162,10 +162,15 @@ __global__ void __launch_bounds__(256) proj_norm_prep_kernel(const T* __restrict
                                                              int inter, float eps, const float* __restrict__ qscale,
                                                              int vnorm, const int* __restrict__ pos,
                                                              const int* __restrict__ slots, T* __restrict__ kc,
-                                                             T* __restrict__ vc, T* __restrict__ q, int BSZ) {
+                                                             T* __restrict__ vc, T* __restrict__ q, int BSZ,
+                                                             T* __restrict__ zrow, int zn) {
+  // zrow: a [T, zn] buffer whose row of this token is cleared (the attention output of a step with
+  // padding rows, which no attention tile writes)
   __shared__ float red[16];
   const long tok = blockIdx.x;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  if (zrow)
+    for (int e = tid; e < zn; e += 256) stf(zrow + tok * zn + e, 0.f);
   const T* r = proj + tok * ld;
   const int slot = kc ? slots[tok] : -1;
   const long blk = slot >= 0 ? slot / BSZ : 0;
@@ -799,15 +804,15 @@ extern "C" int dllm_diff_combine(const float* a, void* out, int f32, long T, int
 extern "C" int dllm_proj_norm_prep(const void* proj, long ld, int f32, int H, int G, int d, int dv, const float* qw,
                                    const float* kw, const float* cos_sin, int tab_w, int rot, int inter, float eps,
                                    const float* qscale, int vnorm, const int* pos, const int* slots, void* kc, void* vc, void* q,
-                                   long T, int BSZ, hipStream_t st) {
+                                   long T, int BSZ, void* zrow, int zn, hipStream_t st) {
   if (T <= 0) return 0;
   if (rot < 0 || rot > d || (rot & 1) || rot > tab_w || H < 1 || G < 1 || H % G) return -1;
   const dim3 grid((unsigned)T);
   if (f32)
     hipLaunchKernelGGL(proj_norm_prep_kernel<float>, grid, dim3(256), 0, st, (const float*)proj, ld, H, G, d, dv, qw, kw, cos_sin,
-                       tab_w, rot, inter, eps, qscale, vnorm, pos, slots, (float*)kc, (float*)vc, (float*)q, BSZ);
+                       tab_w, rot, inter, eps, qscale, vnorm, pos, slots, (float*)kc, (float*)vc, (float*)q, BSZ, (float*)zrow, zn);
   else
     hipLaunchKernelGGL(proj_norm_prep_kernel<u16>, grid, dim3(256), 0, st, (const u16*)proj, ld, H, G, d, dv, qw, kw, cos_sin,
-                       tab_w, rot, inter, eps, qscale, vnorm, pos, slots, (u16*)kc, (u16*)vc, (u16*)q, BSZ);
+                       tab_w, rot, inter, eps, qscale, vnorm, pos, slots, (u16*)kc, (u16*)vc, (u16*)q, BSZ, (u16*)zrow, zn);
   return (int)hipGetLastError();
 }

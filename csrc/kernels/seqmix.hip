@@ -209,12 +209,14 @@ __global__ void __launch_bounds__(256) conv_refill_kernel(const T* __restrict__ 
 }
 
 // ---------------------------------------------------------------- causal conv + SiLU
+// x and y may be the same buffer in a step of single tokens (every output element is written by the
+// thread that alone has read its input), so neither is declared restrict.
 template <typename T>
-__global__ void __launch_bounds__(256) conv_silu_kernel(const T* __restrict__ x, long ldx, const float* __restrict__ w,
+__global__ void __launch_bounds__(256) conv_silu_kernel(const T* x, long ldx, const float* __restrict__ w,
                                                         const float* __restrict__ b, const T* state,
                                                         const int* __restrict__ qstart, const int* __restrict__ qlen,
                                                         const int* __restrict__ ctx, const int* __restrict__ rows,
-                                                        T* __restrict__ y, int C, int K, T* refill, int act) {
+                                                        T* y, int C, int K, T* refill, int act) {
   // act 0: y = silu(b + conv);  act 1: y = x + b + conv (an input convolution ahead of a mixer)
   const int s = blockIdx.y;
   const int n = qlen[s];
@@ -225,23 +227,27 @@ __global__ void __launch_bounds__(256) conv_silu_kernel(const T* __restrict__ x,
   const T* st = state + (long)rows[s] * (K - 1) * C;
   const int step = 4 * gridDim.z;
   const float bias = b[c];
+  float x0 = 0.f;     // the first token's own input (read before its output is stored)
   for (int j = blockIdx.z * 4 + (threadIdx.x >> 6); j < n; j += step) {
     float acc = bias;
-    for (int k = 0; k < K; ++k) {
+    for (int k = 0; k + 1 < K; ++k) {
       const int i = j - (K - 1) + k;
       float u = 0.f;
       if (i >= 0) u = ldf(x + (long)(q0 + i) * ldx + c);
       else if (p0 > 0) u = ldf(st + (long)(K - 1 + i) * C + c);
       acc += w[c * K + k] * u;
     }
-    stf(y + (long)(q0 + j) * C + c, act ? acc + ldf(x + (long)(q0 + j) * ldx + c) : silu_f(acc));
+    const float xj = ldf(x + (long)(q0 + j) * ldx + c);
+    if (j == 0) x0 = xj;
+    acc += w[c * K + K - 1] * xj;
+    stf(y + (long)(q0 + j) * C + c, act ? acc + xj : silu_f(acc));
   }
   // decode steps (`refill` set; every sequence brings one token, which this thread alone has read
   // the slot for): shift the slot's inputs by one and append the token's, in the same launch
   if (refill && n == 1 && K > 1 && blockIdx.z == 0 && (threadIdx.x >> 6) == 0) {
     T* sw = refill + (long)rows[s] * (K - 1) * C + c;
     for (int k = 0; k + 1 < K - 1; ++k) stf(sw + (long)k * C, p0 > 0 ? ldf(sw + (long)(k + 1) * C) : 0.f);
-    stf(sw + (long)(K - 2) * C, ldf(x + (long)q0 * ldx + c));
+    stf(sw + (long)(K - 2) * C, x0);
   }
 }
 

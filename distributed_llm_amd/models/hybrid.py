@@ -642,7 +642,8 @@ class HybridModel:
         the sequence's last inputs."""
         single = meta.host_qlen is None      # a decode step: the convolution refills its slots itself
         y = seqmix.causal_conv_silu(h, L["canon"], L["canon_b"], state, meta.qstart, meta.qlen, meta.ctx,
-                                    meta.state_rows, refill=single, act="residual", all_rows=self._all_rows(h, meta))
+                                    meta.state_rows, refill=single, act="residual", all_rows=self._all_rows(h, meta),
+                                    inplace=single)
         if not single:
             seqmix.conv_state_refill(h, state, meta.qstart, meta.qlen, meta.ctx, meta.state_rows)
         return y
@@ -653,15 +654,17 @@ class HybridModel:
         proj = _mm(x, L["proj"])                                        # q | k | v, or q alone
         rot = m.rot.dims if m.rot is not None else 0
         table = self._table(m) if rot else self._any_table()
+        # a step with padding rows (decode graphs): the prep launch clears the attention output's rows
+        out = None if self._all_rows(x, meta) else torch.empty((x.shape[0], m.heads * m.vdim), dtype=x.dtype, device=x.device)
         q = seqmix.proj_norm_prep(proj, m.heads, m.kv_heads, m.dim, m.vdim, L["qnorm"], L["knorm"], table, rot, True,
                                   self.cfg.rms_eps, L["qscale"], True, positions, meta.slots, k_cache if own else None,
-                                  v_cache if own else None)
+                                  v_cache if own else None, zero_rows=out)
         mfma = seqmix.gqa_use_mfma(q, m.heads, m.kv_heads, m.dim, m.vdim, k_cache.shape[2])
         ts, tt = meta.latent_tiles(1, self.device, seqmix.gqa_tokens_per_tile(m.heads, m.kv_heads, mfma))
         splits = seqmix.gqa_splits(int(ts.numel()), m.kv_heads, meta.max_ctx, m.window, m.keep_first) if mfma else 1
         o = seqmix.paged_gqa_attention(q, k_cache, v_cache, meta.block_tables, meta.qstart, meta.qlen, meta.ctx, ts, tt,
                                        None, mfma, splits, window=m.window, keep_first=m.keep_first, sink=m.sink,
-                                       all_rows=self._all_rows(x, meta))
+                                       all_rows=self._all_rows(x, meta), out=out)
         return _mm(o, L["o"])
 
     @staticmethod

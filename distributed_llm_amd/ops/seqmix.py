@@ -51,18 +51,22 @@ def norm_resadd(y: torch.Tensor, w: torch.Tensor, eps: float, x: torch.Tensor,
 
 
 def causal_conv_silu(x, w, b, conv_state, qstart, qlen, ctx, rows, refill: bool = False,
-                     act: str = "silu", all_rows: bool = False) -> torch.Tensor:
+                     act: str = "silu", all_rows: bool = False, inplace: bool = False) -> torch.Tensor:
     """``refill``: the step brings at most one token per sequence (a decode step) and the kernel also
     moves each token's input into its slot; otherwise the slot is left to ``conv_state_refill`` or
     to the scan.  ``act`` "residual": no activation, y = x + the convolution (an input convolution
     ahead of a mixer).  ``all_rows``: every row of x belongs to a sequence (a step of prompt portions
-    without padding), so the output needs no zero fill."""
+    without padding), so the output needs no zero fill.  ``inplace`` (with ``refill``, x [T, C]
+    contiguous): the output overwrites x; rows of no sequence keep their input."""
     ext = _native(x)
     if ext is None:
         y = ref.causal_conv_silu(x, w, b, conv_state, qstart, qlen, ctx, rows, act)
         if refill:
             ref.conv_state_refill(x, conv_state, qstart, qlen, ctx, rows)
         return y
+    if inplace and refill and x.is_contiguous() and x.shape[1] == w.shape[0]:
+        ext.causal_conv_silu(x, w, b, conv_state, qstart, qlen, ctx, rows, x, True, 0 if act == "silu" else 1)
+        return x
     # rows of no sequence (graph padding) stay zero, never stale memory
     y = (torch.empty if all_rows else torch.zeros)((x.shape[0], w.shape[0]), dtype=x.dtype, device=x.device)
     ext.causal_conv_silu(x, w, b, conv_state, qstart, qlen, ctx, rows, y, bool(refill), 0 if act == "silu" else 1)
@@ -299,7 +303,7 @@ def gqa_splits(n_tiles: int, kv_heads: int, max_ctx: int, window: int = 0, keep_
 def paged_gqa_attention(q, k_cache, v_cache, block_tables, qstart, qlen, ctx, tile_seq, tile_tok0,
                         gate: Optional[torch.Tensor] = None, mfma: bool = False, splits: int = 1, window: int = 0,
                         out_f32: bool = False, keep_first: int = 0, sink: float = 0.0,
-                        all_rows: bool = False) -> torch.Tensor:
+                        all_rows: bool = False, out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Causal softmax attention over paged keys / values of any head widths (f32 scores, online
     softmax), output times sigmoid(gate).  ``tile_seq`` / ``tile_tok0``: one entry per
     ``gqa_tokens_per_tile(heads, kv_heads, mfma)`` new tokens of a sequence.  ``splits`` > 1
@@ -309,14 +313,16 @@ def paged_gqa_attention(q, k_cache, v_cache, block_tables, qstart, qlen, ctx, ti
     are read as well).  ``sink`` > 0: one more term of score 0 and that weight in every softmax
     denominator, with no value.  A value cache with fewer heads than the key cache is shared by
     neighbouring key heads.  ``out_f32``: the output stays f32 whatever the model dtype.  ``all_rows``:
-    the tiles cover every row of q (no padding rows), so the output needs no zero fill."""
+    the tiles cover every row of q (no padding rows), so the output needs no zero fill.  ``out``: a
+    prepared output [T, heads * vdim] (its padding rows already cleared)."""
     ext = _native(q)
     if ext is None:
         return ref.paged_gqa_attention(q, k_cache, v_cache, block_tables, qstart, qlen, ctx, gate, window, out_f32,
                                        keep_first, sink)
     dv = v_cache.shape[2]
-    out = (torch.empty if all_rows else torch.zeros)((q.shape[0], q.shape[1] * dv),
-                                                     dtype=torch.float32 if out_f32 else q.dtype, device=q.device)
+    if out is None:
+        out = (torch.empty if all_rows else torch.zeros)((q.shape[0], q.shape[1] * dv),
+                                                         dtype=torch.float32 if out_f32 else q.dtype, device=q.device)
     splits = int(splits) if mfma else 1
     part = None
     if splits > 1:
@@ -541,21 +547,24 @@ def ls_resadd_ln(x: torch.Tensor, w: torch.Tensor, b: torch.Tensor, eps: float, 
 
 
 def proj_norm_prep(proj, heads, kv_heads, dim, vdim, qnorm_w, knorm_w, cos_sin, rot_dims, interleaved, eps, qscale,
-                   vnorm, positions, slots, k_cache, v_cache) -> torch.Tensor:
+                   vnorm, positions, slots, k_cache, v_cache, zero_rows: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Attention inputs with the q / k RMS norm taken over the whole projection (all heads together,
     weights of that length) before the rotation; rotary pairs (2i, 2i + 1) when ``interleaved`` else
     (i, i + rot_dims / 2) on the first ``rot_dims`` dims of every head; q times ``qscale[head]`` (f32);
     ``vnorm``: every value head to unit RMS.  proj [T, q | k | v]; k and v go to their page slots
     (k_cache [blocks, kv_heads, block, dim], v_cache [blocks, kv_heads, vdim, block]); ``k_cache``
-    None (a layer that reads another layer's keys and values): proj holds q alone.
-    Returns q [T, heads, dim]."""
+    None (a layer that reads another layer's keys and values): proj holds q alone.  ``zero_rows``
+    [T, n] (the activations' dtype) is cleared in the same launch: the attention output of a step with
+    padding rows.  Returns q [T, heads, dim]."""
     ext = _native(proj)
     if ext is None:
+        if zero_rows is not None:
+            zero_rows.zero_()
         return ref.proj_norm_prep(proj, heads, kv_heads, dim, vdim, qnorm_w, knorm_w, cos_sin, rot_dims, interleaved,
                                   eps, qscale, vnorm, positions, slots, k_cache, v_cache)
     q = torch.empty((proj.shape[0], heads, dim), dtype=proj.dtype, device=proj.device)     # every row is written
     ext.proj_norm_prep(proj, int(heads), int(kv_heads), int(dim), int(vdim), qnorm_w, knorm_w, cos_sin, int(rot_dims),
-                       bool(interleaved), float(eps), qscale, bool(vnorm), positions, slots, k_cache, v_cache, q)
+                       bool(interleaved), float(eps), qscale, bool(vnorm), positions, slots, k_cache, v_cache, q, zero_rows)
     return q
 
 

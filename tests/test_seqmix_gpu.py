@@ -523,7 +523,7 @@ def test_input_convolution(dt, case, C, K):
     x = torch.randn(T, C + 5, device=DEV).to(dt)
     w, b = torch.randn(C, K, device=DEV) * 0.5, torch.zeros(C, device=DEV)
     st1 = torch.randn(len(case[0]), K - 1, C, device=DEV).to(dt)
-    st2 = st1.clone()
+    st2, st3 = st1.clone(), st1.clone()
     single = max(case[0]) <= 1
     got = seqmix.causal_conv_silu(x, w, b, st1, qstart, qlen, ctx, rows, refill=single, act="residual")
     want = ref.causal_conv_silu(x, w, b, st2, qstart, qlen, ctx, rows, act="residual")
@@ -532,6 +532,12 @@ def test_input_convolution(dt, case, C, K):
         seqmix.conv_state_refill(x, st1, qstart, qlen, ctx, rows)
     ref.conv_state_refill(x, st2, qstart, qlen, ctx, rows)
     torch.testing.assert_close(st1.float(), st2.float(), atol=0, rtol=0)
+    if single:      # the same step with the output written over the input
+        xc = x[:, :C].contiguous()
+        out = seqmix.causal_conv_silu(xc, w, b, st3, qstart, qlen, ctx, rows, refill=True, act="residual", inplace=True)
+        assert out.data_ptr() == xc.data_ptr()
+        torch.testing.assert_close(out.float(), want.float(), **tol(dt))
+        torch.testing.assert_close(st3.float(), st2.float(), atol=0, rtol=0)
 
 
 @pytest.mark.parametrize("dt", DTYPES)
@@ -584,8 +590,11 @@ def test_sink_attention_kernels(dt, case, H, G, d, dv, rot, win, keep):
         torch.testing.assert_close(q1.float(), q2.float(), **tol(dt))
         torch.testing.assert_close(kc1.float(), kc2.float(), **tol(dt))
         torch.testing.assert_close(vc1.float(), vc2.float(), **tol(dt))
-        q3 = seqmix.proj_norm_prep(proj, H, G, d, dv, qw, qw, table, rot, inter, 1e-5, qscale, inter, pos, slots, None, None)
+        stale = torch.full((T, H * dv), float("nan"), device=DEV).to(dt)
+        q3 = seqmix.proj_norm_prep(proj, H, G, d, dv, qw, qw, table, rot, inter, 1e-5, qscale, inter, pos, slots, None, None,
+                                   zero_rows=stale)
         torch.testing.assert_close(q3.float(), q2.float(), **tol(dt))
+        assert float(stale.float().abs().max()) == 0.0 if T else True
     meta = AttnMeta(slots=None, block_tables=bt, qstart=qstart, qlen=qlen, ctx=ctx, tile_seq=None, tile_tok0=None,
                     last_idx=None, host_qlen=case[0])
     forms = [False] + ([True] if seqmix.gqa_use_mfma(q2, H, G, d, dv, 16) else [])
