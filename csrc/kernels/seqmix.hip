@@ -251,6 +251,67 @@ __global__ void __launch_bounds__(256) conv_silu_kernel(const T* x, long ldx, co
   }
 }
 
+// The same convolution for prompt portions of bf16 rows of whole 16-byte vectors: a lane owns 8
+// neighbouring channels (one vector), a wave walks a run of CV_RUN consecutive tokens with the last
+// K - 1 input rows in registers, so every input row is loaded once per run (plus K - 1 rows of history
+// at its start) and every output row leaves as one vector store.
+constexpr int CV_RUN = 8;
+template <int K>
+__global__ void __launch_bounds__(256) conv_vec_kernel(const u16* __restrict__ x, long ldx, const float* __restrict__ w,
+                                                       const float* __restrict__ b, const u16* __restrict__ state,
+                                                       const int* __restrict__ qstart, const int* __restrict__ qlen,
+                                                       const int* __restrict__ ctx, const int* __restrict__ rows,
+                                                       u16* __restrict__ y, int C, int act) {
+  const int s = blockIdx.y;
+  const int n = qlen[s];
+  if (n <= 0) return;
+  const int c = (blockIdx.x * 64 + (threadIdx.x & 63)) * 8;
+  if (c >= C) return;
+  const int q0 = qstart[s], p0 = ctx[s] - n;
+  const u16* st = state + (long)rows[s] * (K - 1) * C;
+  float wk[K][8], bias[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    bias[e] = b[c + e];
+#pragma unroll
+    for (int k = 0; k < K; ++k) wk[k][e] = w[(c + e) * K + k];
+  }
+  const int stride = 4 * gridDim.z * CV_RUN;
+  for (int j0 = (blockIdx.z * 4 + (threadIdx.x >> 6)) * CV_RUN; j0 < n; j0 += stride) {
+    float hist[K > 1 ? K - 1 : 1][8];
+#pragma unroll
+    for (int k = 0; k + 1 < K; ++k) {
+      const int i = j0 - (K - 1) + k;
+      uint4 v = make_uint4(0u, 0u, 0u, 0u);
+      if (i >= 0) v = ld16(x + (long)(q0 + i) * ldx + c);
+      else if (p0 > 0) v = ld16(st + (long)(K - 1 + i) * C + c);
+      unpack8(v, hist[k]);
+    }
+    const int jn = min(CV_RUN, n - j0);
+    for (int jj = 0; jj < jn; ++jj) {
+      float cur[8], o[8];
+      unpack8(ld16(x + (long)(q0 + j0 + jj) * ldx + c), cur);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        float acc = bias[e];
+#pragma unroll
+        for (int k = 0; k + 1 < K; ++k) acc += wk[k][e] * hist[k][e];
+        acc += wk[K - 1][e] * cur[e];
+        o[e] = act ? acc + cur[e] : silu_f(acc);
+      }
+      st16(y + (long)(q0 + j0 + jj) * C + c, pack8(o));
+#pragma unroll
+      for (int k = 0; k + 2 < K; ++k)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) hist[k][e] = hist[k + 1][e];
+      if (K > 1) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) hist[K - 2][e] = cur[e];
+      }
+    }
+  }
+}
+
 // ---------------------------------------------------------------- selective scan
 // 16 lanes per channel; lane `sub` owns states sub, sub + 16, ... (NS of them).  Tokens run in
 // groups of 16: the group's B / C rows are staged once per workgroup in LDS (every channel reads the
@@ -724,17 +785,16 @@ __global__ void __launch_bounds__(256) route_topk_kernel(const float* __restrict
                                                          int count, int keep, int smode, int gmode,
                                                          const float* __restrict__ corr, int real, int* __restrict__ ids,
                                                          float* __restrict__ wts, float* __restrict__ idw) {
-  __shared__ float sc_[4][ROUTER_MAX_E];     // scores
-  __shared__ float ch_[4][ROUTER_MAX_E];     // choice scores; -inf: taken
-  __shared__ float gs_[4][ROUTER_MAX_E];     // group scores; -inf: kept (taken out of the running)
-  __shared__ unsigned char ok_[4][ROUTER_MAX_E];
+  // per wave: scores [E], choice scores [E] (-inf: taken), group scores [E], kept-group flags [E bytes]
+  extern __shared__ float rsm[];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int t = blockIdx.x * 4 + wave;
   if (t >= T) return;
-  float* sc = sc_[wave];
-  float* ch = ch_[wave];
-  float* gs = gs_[wave];
-  unsigned char* ok = ok_[wave];
+  const int per_wave = 3 * E + (E + 3) / 4;
+  float* sc = rsm + wave * per_wave;
+  float* ch = sc + E;
+  float* gs = ch + E;
+  unsigned char* ok = reinterpret_cast<unsigned char*>(gs + E);
   const float* z = logits + (long)t * ld;
   if (smode == 0) {
     for (int e = lane; e < E; e += 64) sc[e] = 1.f / (1.f + expf(-z[e]));
@@ -1004,6 +1064,25 @@ extern "C" int dllm_conv_silu(const void* x, long ldx, int f32, const float* w, 
                               int S, int C, int K, int refill, int act, hipStream_t st) {
   if (T <= 0 || S <= 0) return 0;
   if (K < 1 || K > 9) return -1;
+  // prompt portions of bf16 rows made of whole, aligned 16-byte vectors: the vector kernel
+  if (!f32 && !refill && K <= 5 && T >= 4 * S && C % 8 == 0 && ldx % 8 == 0 && ((uintptr_t)x % 16) == 0 &&
+      ((uintptr_t)y % 16) == 0 && ((uintptr_t)state % 16) == 0) {
+    int gzv = (T + 4 * CV_RUN - 1) / (4 * CV_RUN);
+    if (gzv > 256) gzv = 256;
+    const dim3 gv((C / 8 + 63) / 64, S, gzv);
+#define CONV_VEC(KK)                                                                                                       \
+  hipLaunchKernelGGL(conv_vec_kernel<KK>, gv, dim3(256), 0, st, (const u16*)x, ldx, w, b, (const u16*)state, qstart, qlen, ctx, \
+                     rows, (u16*)y, C, act)
+    switch (K) {
+      case 1: CONV_VEC(1); break;
+      case 2: CONV_VEC(2); break;
+      case 3: CONV_VEC(3); break;
+      case 4: CONV_VEC(4); break;
+      default: CONV_VEC(5); break;
+    }
+#undef CONV_VEC
+    return (int)hipGetLastError();
+  }
   int gz = (T + 31) / 32;
   if (gz > 128) gz = 128;
   const dim3 g((C + 63) / 64, S, gz), blk(256);
@@ -1148,7 +1227,9 @@ extern "C" int dllm_route_topk(const float* logits, long ld, int T, int E, int t
   if (E < 1 || E > ROUTER_MAX_E || ld < E || count < 1 || E % count || keep < 1 || keep > count || top < 1 ||
       top > keep * (E / count) || real < 0)
     return -1;
-  hipLaunchKernelGGL(route_topk_kernel, dim3((T + 3) / 4), dim3(256), 0, st, logits, ld, T, E, top, count, keep, smode, gmode,
+  const long lds = 4L * 4 * (3 * E + (E + 3) / 4);     // sized by the outputs: small routers keep every CU full
+  ENSURE_LDS(route_topk_kernel, lds);
+  hipLaunchKernelGGL(route_topk_kernel, dim3((T + 3) / 4), dim3(256), lds, st, logits, ld, T, E, top, count, keep, smode, gmode,
                      corr, real, ids, wts, idw);
   return (int)hipGetLastError();
 }

@@ -514,8 +514,8 @@ def test_ls_resadd_ln(dt, n, terms):
 
 
 @pytest.mark.parametrize("dt", DTYPES)
-@pytest.mark.parametrize("case", CASES)
-@pytest.mark.parametrize("C,K", [(40, 3), (128, 4), (72, 1), (64, 7)])
+@pytest.mark.parametrize("case", CASES + [([300, 2, 41], [5, 0, 16])])
+@pytest.mark.parametrize("C,K", [(40, 3), (128, 4), (72, 1), (64, 7), (1032, 5), (36, 2)])
 def test_input_convolution(dt, case, C, K):
     """y = x + conv(x) without an activation; decode steps refill the slot in the same launch."""
     torch.manual_seed(22)
