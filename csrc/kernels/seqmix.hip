@@ -943,21 +943,24 @@ __global__ void __launch_bounds__(256) ls_resadd_ln_kernel(const T* __restrict__
 template <typename T>
 __global__ void __launch_bounds__(256) glu_act_kernel(const T* __restrict__ gu, long ld, const float* __restrict__ bias,
                                                       int ff, int mode, float limit, float alpha, T* __restrict__ y,
-                                                      long total) {
-  for (long e = (long)blockIdx.x * 256 + threadIdx.x; e < total; e += (long)gridDim.x * 256) {
-    const long r = e / ff;
-    const int c = (int)(e % ff);
-    float g = ldf(gu + r * ld + c), u = ldf(gu + r * ld + ff + c);
-    if (bias) { g += bias[c]; u += bias[ff + c]; }
-    float o;
-    if (mode == 0) {
-      o = silu_f(g) * u;
-    } else {
+                                                      long rows) {
+  // grid: x over the ff columns, y over the rows (strided when there are more rows than the grid is
+  // tall), so that no thread divides
+  const int c = blockIdx.x * 256 + threadIdx.x;
+  if (c >= ff) return;
+  const float bg = bias ? bias[c] : 0.f, bu = bias ? bias[ff + c] : 0.f;
+  for (long r = blockIdx.y; r < rows; r += gridDim.y) {
+    float g = ldf(gu + r * ld + c) + bg, u = ldf(gu + r * ld + ff + c) + bu;
+    float a = 1.f;
+    if (mode != 0) {
       g = fminf(g, limit);
-      u = fminf(fmaxf(u, -limit), limit);
-      o = g / (1.f + expf(-alpha * g)) * (u + 1.f);
+      u = fminf(fmaxf(u, -limit), limit) + 1.f;
+      a = alpha;
     }
-    stf(y + e, o);
+    // the result is rounded to bf16 in bf16 models: the hardware exponential and reciprocal are exact enough there
+    const float den = 1.f + fastexp<T>::f(-a * g);
+    const float sg = sizeof(T) == 2 ? g * __builtin_amdgcn_rcpf(den) : g / den;
+    stf(y + r * (long)ff + c, sg * u);
   }
 }
 
@@ -1294,10 +1297,9 @@ extern "C" int dllm_glu_act(const void* gu, long ld, int f32, const float* bias,
   const long total = rows * ff;
   if (total <= 0) return 0;
   if (mode < 0 || mode > 1) return -1;
-  long nb = (total + 255) / 256;
-  if (nb > 65535 * 16) nb = 65535 * 16;
+  const dim3 grid((unsigned)((ff + 255) / 256), (unsigned)(rows < 2048 ? rows : 2048));
   BY_T(f32,
-       hipLaunchKernelGGL(glu_act_kernel<u16>, dim3((unsigned)nb), dim3(256), 0, st, (const u16*)gu, ld, bias, ff, mode, limit, alpha, (u16*)y, total),
-       hipLaunchKernelGGL(glu_act_kernel<float>, dim3((unsigned)nb), dim3(256), 0, st, (const float*)gu, ld, bias, ff, mode, limit, alpha, (float*)y, total))
+       hipLaunchKernelGGL(glu_act_kernel<u16>, grid, dim3(256), 0, st, (const u16*)gu, ld, bias, ff, mode, limit, alpha, (u16*)y, rows),
+       hipLaunchKernelGGL(glu_act_kernel<float>, grid, dim3(256), 0, st, (const float*)gu, ld, bias, ff, mode, limit, alpha, (float*)y, rows))
   return (int)hipGetLastError();
 }

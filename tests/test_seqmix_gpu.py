@@ -489,9 +489,10 @@ def test_group_router(E, top, count, keep):
 # ----------------------------------------------------------------------------- layer-norm layers, input convolution, wide q/k norms, sink attention
 
 @pytest.mark.parametrize("dt", DTYPES)
-@pytest.mark.parametrize("n", [24, 104, 328, 1000])
+@pytest.mark.parametrize("n", [24, 104, 328, 1000, 4104, 8200])
+@pytest.mark.parametrize("pad", [3, 8])      # rows of y that are, or are not, whole 16-byte vectors
 @pytest.mark.parametrize("terms", ["none", "y", "y+bias", "all", "all-no-gate"])
-def test_ls_resadd_ln(dt, n, terms):
+def test_ls_resadd_ln(dt, n, terms, pad):
     torch.manual_seed(21)
     T = 11
     x1 = torch.randn(T, n, device=DEV) * 3 + 0.7
@@ -499,7 +500,7 @@ def test_ls_resadd_ln(dt, n, terms):
     w, b, ls, bias = (torch.randn(n, device=DEV) for _ in range(4))
     kw = {}
     if terms != "none":
-        kw = dict(y=torch.randn(T, n + 3, device=DEV).to(dt)[:, :n], ls=ls)
+        kw = dict(y=torch.randn(T, n + pad, device=DEV).to(dt)[:, :n], ls=ls)
     if terms in ("y+bias", "all"):
         kw["bias"] = bias
     if terms.startswith("all"):
@@ -543,10 +544,11 @@ def test_input_convolution(dt, case, C, K):
 @pytest.mark.parametrize("dt", DTYPES)
 def test_glu_act(dt):
     torch.manual_seed(23)
-    gu = (torch.randn(33, 2 * 70 + 4, device=DEV) * 3).to(dt)[:, :140]
-    bias = torch.randn(140, device=DEV)
-    for kw in (dict(), dict(bias=bias), dict(bias=bias, mode="clamped", limit=1.5, alpha=1.702), dict(mode="clamped", limit=0.3, alpha=1.0)):
-        torch.testing.assert_close(seqmix.glu_act(gu, **kw).float(), ref.glu_act(gu, **kw).float(), **tol(dt))
+    for ff in (70, 72, 1024):      # 72, 1024: rows of whole 16-byte vectors
+        gu = (torch.randn(33, 2 * ff + 8, device=DEV) * 3).to(dt)[:, :2 * ff]
+        bias = torch.randn(2 * ff, device=DEV)
+        for kw in (dict(), dict(bias=bias), dict(bias=bias, mode="clamped", limit=1.5, alpha=1.702), dict(mode="clamped", limit=0.3, alpha=1.0)):
+            torch.testing.assert_close(seqmix.glu_act(gu, **kw).float(), ref.glu_act(gu, **kw).float(), **tol(dt))
 
 
 @pytest.mark.parametrize("score", ["softmax", "sigmoid"])
