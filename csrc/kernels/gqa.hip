@@ -183,25 +183,29 @@ __global__ void __launch_bounds__(256) proj_norm_prep_kernel(const T* __restrict
   for (int e = tid; e < nk; e += 256) { const float v = ldf(r + nq + e); sk += v * v; }
   const float rq = 1.f / sqrtf(block_sum(sq, red) / (float)nq + eps);
   const float rk = nk ? 1.f / sqrtf(block_sum(sk, red) / (float)nk + eps) : 0.f;   // slot is uniform in the workgroup
-  for (int e = tid; e < nq + nk; e += 256) {
-    const bool is_q = e < nq;
-    const int c = is_q ? e : e - nq;           // column inside q or k
-    const int hh = c / d, i = c % d;
-    const T* x = r + (is_q ? 0 : nq);
-    const float* w = is_q ? qw : kw;
+  // a wave per q / k head, a lane per dim: no index arithmetic beyond adds
+  const int units = H + (nk ? G : 0);
+  for (int un = wave; un < units; un += 4) {
+    const bool is_q = un < H;
+    const int hh = is_q ? un : un - H;
+    const T* x = r + (is_q ? 0 : nq) + hh * d;              // this head's columns
+    const float* w = (is_q ? qw : kw) + hh * d;
     const float sc = is_q ? rq : rk;
-    float v = ldf(x + c) * sc * w[c];
-    if (i < rot) {
-      int j, f;
-      bool first;
-      if (inter) { j = i ^ 1; f = i >> 1; first = !(i & 1); }
-      else { first = i < half; j = first ? i + half : i - half; f = first ? i : i - half; }
-      const float cc = cs[f], sn = cs[half + f];
-      const float pv = ldf(x + c - i + j) * sc * w[c - i + j];
-      v = first ? v * cc - pv * sn : v * cc + pv * sn;
+    const float os = is_q ? qscale[hh] : 1.f;
+    T* dst = is_q ? q + (tok * H + hh) * d : kc + ((blk * G + hh) * BSZ + off) * d;
+    for (int i = lane; i < d; i += 64) {
+      float v = ldf(x + i) * sc * w[i];
+      if (i < rot) {
+        int j, f;
+        bool first;
+        if (inter) { j = i ^ 1; f = i >> 1; first = !(i & 1); }
+        else { first = i < half; j = first ? i + half : i - half; f = first ? i : i - half; }
+        const float cc = cs[f], sn = cs[half + f];
+        const float pv = ldf(x + j) * sc * w[j];
+        v = first ? v * cc - pv * sn : v * cc + pv * sn;
+      }
+      stf(dst + i, v * os);
     }
-    if (is_q) stf(q + (tok * H + hh) * d + i, v * qscale[hh]);
-    else stf(kc + ((blk * G + hh) * BSZ + off) * d + i, v);
   }
   if (slot >= 0) {   // values: a wave per value head
     const T* vv = r + nq + nk;
