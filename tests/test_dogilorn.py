@@ -401,7 +401,7 @@ def test_attention_sharp_far_keys(tmp_path, device, n):
     either side of a page (16) or key-tile (64) border, carries a row; prompt and decoded rows; the
     second layer reads the first one's pages through a narrow window with kept first tokens."""
     cfg = make_cfg([attn(heads=2, kv_heads=1, dim=8, vdim=5, rot=4, scale=3.0, size=500, keep_first=0),
-                    attn(heads=2, kv_heads=1, dim=8, vdim=5, rot=4, scale=2.0, size=33, keep_first=20, kv_from=0)], width=16)
+                    attn(heads=2, kv_heads=1, dim=8, vdim=5, rot=4, scale=2.0, size=33, keep_first=19, kv_from=0)], width=16)
     W = make_weights(cfg, seed=n, qk_gain=2.0)
     eng = engine(write_model(tmp_path / "m", cfg, W), device, torch.float32, tokens=max(256, n + 32))
     t = toks(n + 2, seed=n)

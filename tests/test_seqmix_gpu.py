@@ -570,7 +570,7 @@ def test_route_topk(score, group_score, R, real, top, count, keep):
 @pytest.mark.parametrize("dt", DTYPES)
 @pytest.mark.parametrize("case", CASES + [([40, 3], [90, 130]), ([1, 1], [300, 77]), ([150], [170])])
 @pytest.mark.parametrize("H,G,d,dv,rot,win,keep", [(4, 2, 16, 8, 8, 5, 3), (6, 2, 88, 56, 20, 64, 70), (3, 3, 40, 72, 40, 1, 0),
-                                                   (8, 1, 96, 96, 24, 100, 20), (4, 1, 56, 88, 28, 70, 1), (2, 1, 136, 200, 64, 0, 9),
+                                                   (8, 1, 80, 112, 20, 100, 9), (4, 1, 56, 88, 28, 70, 1), (2, 1, 136, 200, 64, 0, 9),
                                                    (5, 5, 24, 40, 0, 17, 130), (8, 2, 64, 64, 64, 3, 64)])
 def test_sink_attention_kernels(dt, case, H, G, d, dv, rot, win, keep):
     """Prep (norm over the whole q / k projection before an interleaved rotation, unit-RMS values),
