@@ -447,18 +447,22 @@ def dogilorn_config(raw: dict, name: str = "dogilorn") -> HybridConfig:
             raise ValueError(f"unknown mixer type {kind!r}")
         mask = m.get("mask") or {}
         src = m.get("kv_from")
-        mix = MixerSpec("sink_attention", heads=int(m["heads"]), kv_heads=int(m.get("kv_heads", m["heads"])),
-                        dim=int(m["dim"]), vdim=int(m["vdim"]), scale=float(m["scale"]), rot=_rope(m.get("rot")),
+        o = None
+        if src is not None:      # sizes of the keys and values it reads default to their owner's
+            if not 0 <= int(src) < i or layers[int(src)].mixer.kv_from is not None:
+                raise ValueError(f"layer {i}: kv_from must name an earlier attention layer with keys of its own")
+            o = layers[int(src)].mixer
+        mix = MixerSpec("sink_attention", heads=int(m["heads"]),
+                        kv_heads=int(m.get("kv_heads", o.kv_heads if o else m["heads"])),
+                        dim=int(m["dim"]), vdim=int(m.get("vdim", o.vdim if o else m["dim"])), scale=float(m["scale"]),
+                        rot=_rope(m["rot"]) if "rot" in m else (o.rot if o else None),
                         window=int(mask.get("size", 0)), keep_first=int(mask.get("keep_first", 0)), sink=1.0,
                         kv_from=None if src is None else int(src))
         if mix.heads % mix.kv_heads:
             raise ValueError("heads must be a multiple of kv_heads")
         if mix.rot is not None and (mix.rot.dims % 2 or mix.rot.dims > mix.dim):
             raise ValueError("rot.dims must be even and at most dim")
-        if mix.kv_from is not None:
-            if not 0 <= mix.kv_from < i or layers[mix.kv_from].mixer.kv_from is not None:
-                raise ValueError(f"layer {i}: kv_from must name an earlier attention layer with keys of its own")
-            o = layers[mix.kv_from].mixer
+        if o is not None:
             if (o.kv_heads, o.dim, o.vdim, o.rot) != (mix.kv_heads, mix.dim, mix.vdim, mix.rot):
                 raise ValueError(f"layer {i}: the layer it takes keys and values from has other head sizes or rotation")
         f = L.get("mlp")

@@ -442,6 +442,11 @@ def test_greedy_generation(full_model, device):
     for p, o in zip(prompts, outs):
         assert o.error is None
         assert o.token_ids == orc.greedy(p, W, cfg, 12)
+    # the sampler on this model's logits: in range, and the same draw for the same seed
+    sp = SamplingParams(max_new_tokens=8, temperature=0.9, top_p=0.9, top_k=20, seed=7, ignore_eos=True)
+    a = [o.token_ids for o in eng.generate(prompts[:2], sp)]
+    b = [o.token_ids for o in eng.generate(prompts[:2], sp)]
+    assert a == b and all(len(t) == 8 and all(0 <= x < cfg["vocab"] for x in t) for t in a)
 
 
 def test_replay_command_line(full_model, tmp_path):
