@@ -4,7 +4,11 @@ residual update, squared-ReLU experts (csrc/kernels/seqmix.hip, latent.hip, moe.
 attention over pages with an optional window and shared value heads, its input kernels (unit-RMS or
 weighted q/k norms, one or two score maps a head) and the gated delta rule (gqa.hip, delta.hip); the
 Mamba-2 and mLSTM recurrences (outer_scan.hip); PolyNorm, the group-limited sigmoid router, the
-dense form of SwiGLU experts and the logit soft cap.
+dense form of SwiGLU experts and the logit soft cap; for pre-norm layer-norm models the sublayer
+tail with layer scale and the next layer norm in one launch, an input convolution without activation,
+attention inputs normed over the whole q / k projection, kept first keys and a softmax sink in the
+paged attention, gated activations with clamps, and top-k routing with softmax scores, a correction
+on the choice and identity experts.
 
 Same dispatch rule as the rest of the op library: GPU tensors run the HIP kernel (or raise when the
 extension is missing), CPU tensors the torch reference.  Every kernel takes bf16 or f32 activations
